@@ -1,0 +1,155 @@
+/*
+ * mi355_fp8.h - C ABI of libmi355fp8.so: hand-written gfx950 (MI355X) kernels for
+ * LightLLM's block-FP8 W8A8 linear path.
+ *
+ * Plain C: pointers are device pointers unless a comment says "host"; sizes and
+ * strides are in ELEMENTS of the tensor they describe; `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).  No entry point allocates or
+ * frees device memory, synchronises the host with the device, or keeps mutable
+ * global state, so all of them may be called under HIP graph capture and from
+ * several host threads at once.  Workspaces are caller-owned.
+ *
+ * Every function returns 0 on success or a negative MI355_E* code; nothing is
+ * launched when a precondition fails.  mi355_error_string() names the code.
+ *
+ * Paths in the citations are relative to the reference tree (LightLLM v1.2.0).
+ */
+#ifndef MI355_FP8_H
+#define MI355_FP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_OK 0
+#define MI355_EINVAL -1        /* a size or enum argument is out of range */
+#define MI355_ESHAPE -2        /* shapes/strides break a precondition the reference asserts */
+#define MI355_EALIGN -3        /* a pointer or leading dimension is not aligned as the kernel needs */
+#define MI355_EWORKSPACE -4    /* workspace missing or smaller than *_workspace_bytes() */
+#define MI355_ELAUNCH -5       /* the HIP runtime refused the launch (hipGetLastError() != hipSuccess) */
+#define MI355_EUNSUPPORTED -6  /* valid request that no kernel variant covers */
+
+const char *mi355_error_string(int code);
+
+/* Device facts the host side sizes launches and rooflines with.
+ * out[0]=compute units, out[1]=max engine clock kHz, out[2]=LDS bytes per workgroup (opt-in max),
+ * out[3]=L2 bytes, out[4]=memory clock kHz, out[5]=memory bus width bits, out[6]=1 if the device is gfx950.
+ * `device` < 0 means the current device. */
+int mi355_device_info(int device, int64_t out[8]);
+
+/* ---------------------------------------------------------------------------
+ * per_token_group_quant_fp8
+ * replaces: lightllm_per_token_group_quant_fp8 + _per_token_group_quant_fp8
+ *           (lightllm/common/basemodel/triton_kernel/quantization/fp8act_quant_kernel.py:18-113)
+ *
+ * x  bf16 [M,K] contiguous           (asserted there at :81)
+ * q  e4m3fn bytes [M,K] contiguous
+ * s  fp32, element (m,g) at s[m*s_stride_m + g*s_stride_g], g < K/group
+ *    row-major (K/group, 1) and column-major (1, ld) are both what the reference
+ *    writes (:37-42); any pair of strides is accepted.
+ * group must be 128 and divide K (:80); eps is the floor on the group amax (:55).
+ * Arithmetic: s = max(amax,eps)/448 and q = e4m3fn_rtne(clamp(x/s,+-448)) with
+ * IEEE fp32 division results, bit for bit.
+ */
+int mi355_group_quant_fp8(const void *x, void *q, float *s, int64_t M, int64_t K, int32_t group, float eps,
+                          int64_t s_stride_m, int64_t s_stride_g, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * weight_quant (load-time 128x128 block quantizer)
+ * replaces: mm_weight_quant / weight_quant_kernel
+ *           (.../quantization/fp8w8a8_block_quant_kernel.py:7-42)
+ *
+ * w bf16 [N,K] contiguous; q e4m3fn [N,K]; s fp32 [ceil(N/128), ceil(K/128)] contiguous.
+ * Keeps the reference's quirk: the stored scale is amax/448 while values are
+ * divided by (scale + 1e-6), without clamp (:22-24).  `w_dtype`: 0 = bf16, 1 = fp32, 2 = fp16.
+ */
+int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float *s, int64_t N, int64_t K,
+                                 int32_t block, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * w8a8_block_fp8_matmul
+ * replaces: w8a8_block_fp8_matmul + _block_scaled_block_gemm
+ *           (.../quantization/fp8w8a8_block_gemm_kernel.py:24-84, 127-192)
+ *
+ * C[m,n] = bf16( sum_kb ( sum_{k in kb} A[m,k]*B[k,n] ) * As[m,kb] * Bs[kb, n/block_n] ), fp32 accumulation.
+ *
+ * A   e4m3fn [M,K], row stride lda, unit column stride (the reference asserts A contiguous, :152)
+ * B   e4m3fn logical [K,N]: element (k,n) at B[k*ldb_k + n*ldb_n].  The reference passes the
+ *     transposed view of an [N,K] weight, i.e. ldb_k = 1, ldb_n = K (common/quantization/w8a8.py:442);
+ *     that layout takes the MFMA kernels, any other pair of strides takes a slow generic kernel.
+ * As  fp32 [M, K/block_k]   element (m,kb) at As[m*as_m + kb*as_k]
+ * Bs  fp32 [K/block_k, ceil(N/block_n)] element (kb,nb) at Bs[kb*bs_k + nb*bs_n]   (w8a8.py:443: strides (1, K/128))
+ * C   bf16 [M,N], row stride ldc, unit column stride (:152)
+ * block_n = block_k = 128.
+ *
+ * `variant` picks the kernel: MI355_GEMM_AUTO applies the built-in shape table; the others force
+ * one (for tests and tuning).  Split-K variants need `ws` of at least
+ * mi355_block_fp8_gemm_workspace_bytes() bytes, whose first MI355_WS_COUNTER_BYTES must be zero
+ * on the first call; the kernels leave them zero again, so one zero-initialised buffer serves every call
+ * issued in order on one stream.
+ */
+#define MI355_GEMM_AUTO 0
+#define MI355_GEMM_TILE256 1     /* 256x256x128 CTA tile, 8 waves, LDS double buffer: compute-bound M */
+#define MI355_GEMM_TILE128 2     /* 128x128x128 CTA tile, 4 waves: mid M or few tiles */
+#define MI355_GEMM_SKINNY 3      /* weight-streaming split-K, M <= 64 */
+#define MI355_GEMM_GENERIC 4     /* any strides, no MFMA; correctness fallback */
+#define MI355_GEMM_TILE256x128 5 /* 256x128x128 CTA tile, 8 waves */
+
+#define MI355_WS_COUNTER_BYTES 65536
+
+size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant);
+
+int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C, int64_t M,
+                         int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                         int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int32_t block_n,
+                         int32_t block_k, void *ws, size_t ws_bytes, int32_t variant, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * moe_align_fused / moe_align2 : routing tables for the grouped GEMM
+ * replaces: moe_align_fused (lightllm/common/basemodel/triton_kernel/fused_moe/grouped_fused_moe.py:388-396)
+ *           moe_align2      (same file :399-477)
+ *
+ * topk_ids int32 [num_pairs] (flattened [tokens, topk]); topk_weights fp32 [num_pairs];
+ * expert_to_token_index int32 [E, num_pairs]; expert_to_weight fp32 [E, num_pairs]; expert_token_num int32 [E].
+ * Within an expert, pair indices come out in ascending order for every size (the reference only
+ * guarantees that below 129 tokens, :391-395).
+ */
+int mi355_moe_align_fused(const int32_t *topk_ids, const float *topk_weights, int64_t num_pairs,
+                          int32_t num_experts, int32_t *expert_to_token_index, float *expert_to_weight,
+                          int32_t *expert_token_num, void *stream);
+
+/* rows of the schedule table: min(num_pairs, ceil((num_pairs + E*(block_m-1)) / block_m))  (:457-458) */
+int64_t mi355_moe_align2_rows(int64_t num_pairs, int32_t num_experts, int32_t block_m);
+
+/* table int32 [rows,3] = (expert, m_index, token_start); padding rows get expert = -1 (:439-446). */
+int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32_t block_m, int64_t rows,
+                     int32_t *table, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * grouped_matmul, fp8 128x128-block branch
+ * replaces: grouped_matmul_kernel + the launch in grouped_matmul
+ *           (.../fused_moe/grouped_fused_moe.py:480-728, 925-988), gather/scatter form
+ *
+ * For each schedule row (e, mi, start) and j in [mi*block_m, min((mi+1)*block_m, expert_token_num[e])):
+ *     idx = expert_to_token_index[e*num_pairs + j];  row = idx / topk_num
+ *     out[idx, :] = bf16( blockscaled(Xq[row,:] . W[e]^T) * (mul_routed_weight ? expert_to_weight[e*num_pairs+j] : 1) )
+ * Xq e4m3fn [T,K] contiguous, Xs fp32 [T,K/128] contiguous (the activation quantizer's output);
+ * W e4m3fn [E,N,K] contiguous; Ws fp32 [E, ceil(N/128), K/128] contiguous; out bf16 [num_pairs, N] contiguous.
+ * block_m must be one the library was built for: 16, 32, 64 or 128 (mi355_grouped_block_m() suggests one).
+ */
+int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K);
+
+int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                 const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                 const int32_t *expert_token_num, const int32_t *table, int64_t table_rows,
+                                 int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
+                                 int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
+                                 void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_FP8_H */

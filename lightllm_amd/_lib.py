@@ -1,0 +1,111 @@
+"""ctypes binding of libmi355fp8.so (the C ABI declared in include/mi355_fp8.h)."""
+import ctypes
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmi355fp8.so")
+
+GEMM_AUTO, GEMM_TILE256, GEMM_TILE128, GEMM_SKINNY, GEMM_GENERIC, GEMM_TILE256x128 = 0, 1, 2, 3, 4, 5
+WS_COUNTER_BYTES = 65536
+
+_c = ctypes
+_vp, _i64, _i32, _f32, _sz = _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_float, _c.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/mi355_fp8.h
+SIGNATURES = {
+    "mi355_error_string": (_c.c_char_p, [_c.c_int]),
+    "mi355_device_info": (_c.c_int, [_c.c_int, _c.POINTER(_i64)]),
+    "mi355_group_quant_fp8": (_c.c_int, [_vp, _vp, _vp, _i64, _i64, _i32, _f32, _i64, _i64, _vp]),
+    "mi355_block_weight_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp]),
+    "mi355_block_fp8_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "mi355_block_fp8_gemm": (
+        _c.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
+         _vp, _sz, _i32, _vp],
+    ),
+    "mi355_moe_align_fused": (_c.c_int, [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp]),
+    "mi355_moe_align2_rows": (_i64, [_i64, _i32, _i32]),
+    "mi355_moe_align2": (_c.c_int, [_vp, _i32, _i32, _i64, _vp, _vp]),
+    "mi355_grouped_block_m": (_i32, [_i64, _i32, _i64, _i64]),
+    "mi355_grouped_block_fp8_gemm": (
+        _c.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp],
+    ),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+class Mi355Error(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """Loads the HIP library; there is no fallback path when it is missing."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise Mi355Error(
+                        f"{LIB_PATH} is missing: build it with `python -m lightllm_amd.build` "
+                        "(hipcc, gfx950). lightllm_amd has no CPU or eager fallback."
+                    )
+                handle = ctypes.CDLL(LIB_PATH)
+                for name, (res, args) in SIGNATURES.items():
+                    fn = getattr(handle, name)
+                    fn.restype = res
+                    fn.argtypes = args
+                _lib = handle
+    return _lib
+
+
+def check(code: int, what: str) -> None:
+    """Re-raise a negative C-ABI status as the Python error the reference would raise."""
+    if code == 0:
+        return
+    msg = lib().mi355_error_string(code).decode()
+    if code in (-2,):
+        raise AssertionError(f"{what}: {msg}")
+    if code in (-1, -3, -4, -6):
+        raise ValueError(f"{what}: {msg}")
+    raise Mi355Error(f"{what}: {msg}")
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise Mi355Error("lightllm_amd operators run on the GPU only; got a CPU tensor")
+
+
+_workspaces = {}
+
+
+def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Per (device, stream) scratch for split-K launches: zero-initialised once, grown on demand.
+
+    The kernels leave the counter words zero, so the buffer is never cleared again.  Growing allocates, so
+    callers that capture HIP graphs must run each shape once before capturing (as with any torch allocator use).
+    """
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr(device))
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        size = max(nbytes, WS_COUNTER_BYTES + (32 << 20))
+        buf = torch.zeros(size, dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def device_info(device: int = -1) -> dict:
+    out = (_i64 * 8)()
+    check(lib().mi355_device_info(device, out), "mi355_device_info")
+    keys = ["compute_units", "clock_khz", "lds_bytes", "l2_bytes", "mem_clock_khz", "mem_bus_bits", "is_gfx950", "hbm_bytes"]
+    return dict(zip(keys, [int(v) for v in out]))

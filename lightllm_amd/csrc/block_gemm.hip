@@ -1,0 +1,290 @@
+// Host side of the block-scaled FP8 GEMM entry points: argument checks, kernel choice, launches.
+#include <mutex>
+
+#include "gemm_tile.hpp"
+
+namespace mi355 {
+
+// Correctness fallback for layouts the MFMA kernels do not take (B not K-contiguous, K not a multiple of
+// 128, unaligned leading dimensions).  One thread per output element, same per-block arithmetic.
+__device__ __forceinline__ float e4m3_to_f32(uint8_t b) {
+    const uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+    const uint32_t e = (b >> 3) & 0xfu, m = b & 7u;
+    float v;
+    if (e == 0) v = (float)m * 0.001953125f;  // m * 2^-9
+    else v = as_f32(((e + 120u) << 23) | (m << 20));
+    return as_f32(as_u32(v) | sign);
+}
+
+__global__ __launch_bounds__(256) void block_fp8_gemm_generic_kernel(
+    const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ As,
+    const float *__restrict__ Bs, uint16_t *__restrict__ C, int M, int N, int K, int64_t lda, int64_t ldb_k,
+    int64_t ldb_n, int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int block_n, int block_k) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)M * N) return;
+    const int m = (int)(idx / N), n = (int)(idx % N);
+    float acc = 0.f;
+    int kb = 0;
+    for (int k0 = 0; k0 < K; k0 += block_k, ++kb) {
+        const int k1 = min(k0 + block_k, K);
+        float d = 0.f;
+        for (int k = k0; k < k1; ++k) d += e4m3_to_f32(A[m * lda + k]) * e4m3_to_f32(B[k * ldb_k + n * ldb_n]);
+        acc += d * As[m * as_m + kb * as_k] * Bs[kb * bs_k + (n / block_n) * bs_n];
+    }
+    C[m * ldc + n] = (uint16_t)f32_to_bf16_bits(acc);
+}
+
+constexpr int kMaxLds = 160 * 1024;  // LDS per workgroup on gfx950
+
+template <typename KernelT>
+static hipError_t allow_lds(KernelT kernel, int bytes) {
+    // Raising the dynamic-LDS ceiling is a per-function host-side setting; it enqueues nothing.
+    return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
+static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
+    using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
+    auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE>;
+    const int KB = a.K / kBlockK;
+    const int lds_bytes = Cfg::lds_bytes(KB);
+    if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] { attr_err = allow_lds(kernel, kMaxLds); });
+    if (attr_err != hipSuccess) return MI355_ELAUNCH;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::kThreads), lds_bytes, st, a);
+    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+static int launch_dense(GemmArgs &a, hipStream_t st) {
+    a.tiles_m = (a.M + BM - 1) / BM;
+    a.tiles_n = (a.N + BN - 1) / BN;
+    a.total_tiles = a.tiles_m * a.tiles_n;
+    a.blocks_per_xcd = (a.total_tiles + 7) / 8;
+    return launch_tile<BM, BN, WM, WN, NSTAGE, kDense>(a, a.blocks_per_xcd * 8, st);
+}
+
+// Weight-streaming launch for M <= 64: tiles BM x 64, deep DMA ring, K split so that about one CTA per CU
+// streams a long run of weight bytes.
+constexpr int kSkinnyBN = 64;
+constexpr int kSkinnyStages = 8;
+
+static int skinny_bm(int64_t M) { return M <= 16 ? 16 : (M <= 32 ? 32 : 64); }
+
+static int skinny_splits(int64_t N, int64_t K, int cus) {
+    const int tiles_n = (int)((N + kSkinnyBN - 1) / kSkinnyBN);
+    const int KB = (int)(K / kBlockK);
+    int splits = (cus + tiles_n - 1) / tiles_n;        // reach at least one CTA per CU
+    const int max_splits = KB / 8 > 0 ? KB / 8 : 1;     // keep at least 8 K steps per CTA
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    return splits;
+}
+
+template <int BM>
+static int launch_skinny(GemmArgs &a, int splits, void *ws, hipStream_t st) {
+    constexpr int BN = kSkinnyBN;
+    a.tiles_m = 1;
+    a.tiles_n = (a.N + BN - 1) / BN;
+    a.total_tiles = a.tiles_n;
+    if (splits <= 1) {
+        a.blocks_per_xcd = (a.total_tiles + 7) / 8;
+        return launch_tile<BM, BN, 1, 4, kSkinnyStages, kDense>(a, a.blocks_per_xcd * 8, st);
+    }
+    a.splits = splits;
+    a.counters = (uint32_t *)ws;
+    a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+    return launch_tile<BM, BN, 1, 4, kSkinnyStages, kSplitK>(a, a.total_tiles * splits, st);
+}
+
+static int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n) {
+    return ldb_k == 1 && K % kBlockK == 0 && lda % 16 == 0 && ldb_n % 16 == 0 && ((uintptr_t)A & 15) == 0 &&
+           ((uintptr_t)B & 15) == 0;
+}
+
+static int pick_variant(int64_t M, int64_t N, int cus) {
+    if (M <= 64) return MI355_GEMM_SKINNY;
+    const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
+    if (t256 >= (int64_t)cus * 3 / 4) return MI355_GEMM_TILE256;
+    return MI355_GEMM_TILE128;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, 256);
+    if (variant != MI355_GEMM_SKINNY || M > 64 || K % kBlockK != 0) return 0;
+    // sized for the largest split any device would pick, so the figure does not depend on the device
+    const int64_t tiles = (N + kSkinnyBN - 1) / kSkinnyBN;
+    int64_t max_splits = K / kBlockK / 8;
+    if (max_splits < 1) max_splits = 1;
+    if (tiles * 4 > MI355_WS_COUNTER_BYTES) return 0;
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * max_splits * skinny_bm(M) * kSkinnyBN * 4;
+}
+
+extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
+                                    int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n,
+                                    int32_t block_n, int32_t block_k, void *ws, size_t ws_bytes, int32_t variant,
+                                    void *stream) {
+    if (M < 0 || N < 0 || K < 0) return MI355_EINVAL;
+    if (block_n != kBlockN || block_k != kBlockK) return MI355_EUNSUPPORTED;
+    if (M == 0 || N == 0) return MI355_OK;
+    if (K == 0) return MI355_ESHAPE;
+    if (!A || !B || !As || !Bs || !C) return MI355_EINVAL;
+    if (lda < K || ldc < N) return MI355_ESHAPE;
+    if (M >= (1ll << 31) || N >= (1ll << 31) || K >= (1ll << 31)) return MI355_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int cus = device_cus();
+
+    const bool fast = fast_layout_ok(A, B, K, lda, ldb_k, ldb_n) &&
+                      // 32-bit byte offsets inside a tile / scale column
+                      256 * lda < (1ll << 32) && 256 * ldb_n < (1ll << 32) && 256 * as_m * 4 < (1ll << 32) &&
+                      as_m >= 0 && as_k >= 0;
+    if (variant == MI355_GEMM_AUTO) variant = fast ? pick_variant(M, N, cus) : MI355_GEMM_GENERIC;
+    if (variant != MI355_GEMM_GENERIC && !fast) return MI355_EALIGN;
+
+    if (variant == MI355_GEMM_GENERIC) {
+        const int64_t blocks = (M * N + 255) / 256;
+        if (blocks >= (1ll << 31)) return MI355_EUNSUPPORTED;
+        hipLaunchKernelGGL(block_fp8_gemm_generic_kernel, dim3((uint32_t)blocks), dim3(256), 0, st,
+                           (const uint8_t *)A, (const uint8_t *)B, As, Bs, (uint16_t *)C, (int)M, (int)N, (int)K, lda,
+                           ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n, (int)block_n, (int)block_k);
+        return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+    }
+
+    GemmArgs a = {};
+    a.X = (const uint8_t *)A;
+    a.W = (const uint8_t *)B;
+    a.Xs = As;
+    a.Ws = Bs;
+    a.C = (uint16_t *)C;
+    a.M = (int)M;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.ldx = lda;
+    a.ldw = ldb_n;
+    a.ldc = ldc;
+    a.xs_m = as_m;
+    a.xs_k = as_k;
+    a.ws_n = bs_n;
+    a.ws_k = bs_k;
+    a.vec_store = (((uintptr_t)C & 15) == 0 && ldc % 8 == 0 && N % 8 == 0) ? 1 : 0;
+
+    switch (variant) {
+        case MI355_GEMM_TILE256:
+            return launch_dense<256, 256, 2, 4, 2>(a, st);
+        case MI355_GEMM_TILE256x128:
+            return launch_dense<256, 128, 2, 4, 3>(a, st);
+        case MI355_GEMM_TILE128:
+            return launch_dense<128, 128, 2, 2, 2>(a, st);
+        case MI355_GEMM_SKINNY: {
+            if (M > 64) return MI355_EUNSUPPORTED;
+            const int splits = skinny_splits(N, K, cus);
+            if (splits > 1) {
+                const size_t need = (size_t)MI355_WS_COUNTER_BYTES +
+                                    (size_t)((N + kSkinnyBN - 1) / kSkinnyBN) * splits * skinny_bm(M) * kSkinnyBN * 4;
+                if (!ws || ws_bytes < need || ((uintptr_t)ws & 15)) return MI355_EWORKSPACE;
+                if (((N + kSkinnyBN - 1) / kSkinnyBN) * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
+            }
+            switch (skinny_bm(M)) {
+                case 16: return launch_skinny<16>(a, splits, ws, st);
+                case 32: return launch_skinny<32>(a, splits, ws, st);
+                default: return launch_skinny<64>(a, splits, ws, st);
+            }
+        }
+        default:
+            return MI355_EINVAL;
+    }
+}
+
+extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K) {
+    (void)N;
+    (void)K;
+    if (num_experts <= 0) return 64;
+    const int64_t avg = num_pairs / num_experts;
+    if (avg <= 16) return 16;
+    if (avg <= 32) return 32;
+    if (avg <= 64) return 64;
+    return 128;
+}
+
+extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                            const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                            const int32_t *expert_token_num, const int32_t *table,
+                                            int64_t table_rows, int32_t block_m, int64_t num_pairs,
+                                            int64_t num_tokens, int32_t num_experts, int32_t topk_num, int64_t N,
+                                            int64_t K, int32_t mul_routed_weight, void *out, void *stream) {
+    if (num_pairs < 0 || num_tokens < 0 || num_experts <= 0 || topk_num <= 0 || N < 0 || K < 0 || table_rows < 0)
+        return MI355_EINVAL;
+    if (num_pairs == 0 || N == 0 || table_rows == 0) return MI355_OK;
+    if (!Xq || !Xs || !W || !Ws || !expert_to_token_index || !expert_to_weight || !expert_token_num || !table || !out)
+        return MI355_EINVAL;
+    if (K == 0 || K % kBlockK != 0) return MI355_ESHAPE;
+    if (((uintptr_t)Xq & 15) || ((uintptr_t)W & 15)) return MI355_EALIGN;
+    if (num_tokens * K >= (1ll << 32) || 256 * K >= (1ll << 32) || num_tokens * (K / kBlockK) * 4 >= (1ll << 32) ||
+        N >= (1ll << 31) || num_pairs >= (1ll << 31))
+        return MI355_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t KB = K / kBlockK, NB = (N + kBlockN - 1) / kBlockN;
+
+    GemmArgs a = {};
+    a.X = (const uint8_t *)Xq;
+    a.W = (const uint8_t *)W;
+    a.Xs = Xs;
+    a.Ws = Ws;
+    a.C = (uint16_t *)out;
+    a.M = (int)num_pairs;
+    a.N = (int)N;
+    a.K = (int)K;
+    a.ldx = K;
+    a.ldw = K;
+    a.ldc = N;
+    a.xs_m = KB;
+    a.xs_k = 1;
+    a.ws_n = KB;
+    a.ws_k = 1;
+    a.vec_store = (((uintptr_t)out & 15) == 0 && N % 8 == 0) ? 1 : 0;
+    a.table = table;
+    a.e2t_index = expert_to_token_index;
+    a.e2t_weight = expert_to_weight;
+    a.e_num = expert_token_num;
+    a.w_e = N * K;
+    a.ws_e = NB * KB;
+    a.num_pairs = (int)num_pairs;
+    a.topk = topk_num;
+    a.mul_weight = mul_routed_weight ? 1 : 0;
+    a.tiles_m = (int)table_rows;
+
+    auto finish = [&](int BN) {
+        a.tiles_n = (int)((N + BN - 1) / BN);
+        a.total_tiles = a.tiles_m * a.tiles_n;
+        a.blocks_per_xcd = (a.total_tiles + 7) / 8;
+        return a.blocks_per_xcd * 8;
+    };
+    if ((int64_t)table_rows * ((N + 127) / 128) >= (1ll << 31)) return MI355_EUNSUPPORTED;
+    switch (block_m) {
+        case 16: return launch_tile<16, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
+        case 32: return launch_tile<32, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
+        case 64: return launch_tile<64, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
+        case 128: return launch_tile<128, 128, 2, 2, 2, kGrouped>(a, finish(128), st);
+        default: return MI355_EINVAL;
+    }
+}

@@ -1,0 +1,86 @@
+// Shared device helpers for the gfx950 block-FP8 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355_fp8.h"
+
+namespace mi355 {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kBlockK = 128;  // K extent of one scale step (= the 128x128 weight block, the 1x128 activation group)
+constexpr int kBlockN = 128;
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// fp32 -> bf16 bits, round to nearest even (finite inputs).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = as_u32(f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    uint32_t a = as_u32(lo), b = as_u32(hi);
+    a += 0x7fffu + ((a >> 16) & 1u);
+    b += 0x7fffu + ((b >> 16) & 1u);
+    return (a >> 16) | (b & 0xffff0000u);
+}
+
+// D(16x16, fp32) = A(16x128, e4m3) * B(128x16, e4m3) + C on the CDNA4 matrix core.
+// Lane l feeds row/col (l % 16) and the 32 K-bytes numbered (l / 16); both operands use the same
+// K numbering, so any consistent placement of K bytes in the two registers gives the same dot product.
+// D: lane l holds column (l % 16), rows 4*(l/16) + 0..3.
+// Format selectors 0/0 = e4m3 for both operands; block-scale operands 0/0 select the unscaled instruction.
+__device__ __forceinline__ v4f mfma_16x16x128_fp8(v8i a, v8i b, v4f c) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+// Byte address of a __shared__ object inside the workgroup's LDS allocation.
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
+// Asynchronous 16-byte-per-lane copy global -> LDS that bypasses the register file.
+// Lane l's 16 bytes at (gbase + voff) land at LDS byte (lds_base + 16*l): one call fills 1 KiB.
+// lds_base and gbase are wave-uniform.  Completion is tracked by vmcnt; the compiler does not
+// see the LDS write, so the caller orders it with wait_vmcnt<>() and a workgroup barrier.
+__device__ __forceinline__ void dma_g2l_b128(uint32_t lds_base, const void *gbase, uint32_t voff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %2"
+        :
+        : "s"(lds_base), "v"(voff), "s"(gbase)
+        : "memory");
+}
+// Same with 4 bytes per lane (256 B per call), used for scale vectors.
+__device__ __forceinline__ void dma_g2l_b32(uint32_t lds_base, const void *gbase, uint32_t voff) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dword %1, %2"
+        :
+        : "s"(lds_base), "v"(voff), "s"(gbase)
+        : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    // gfx9 encoding of s_waitcnt: vmcnt low bits [3:0], high bits [15:14]; expcnt [6:4]=7, lgkmcnt [11:8]=15 (no wait).
+    __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
+}
+
+// 16B-chunk swizzle for LDS tiles with 128-byte rows (8 chunks per row): physical chunk = logical ^ swz(row).
+// For 16 consecutive rows read at one logical chunk the (row parity, physical chunk) pairs are all
+// distinct, and for 8 consecutive rows the physical chunks are all distinct, so a ds_read_b128 of a
+// 16-row operand slice is bank-conflict free whether the LDS serves 128 or 256 bytes per clock.
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row & 7u) ^ ((row >> 3) & 1u); }
+
+}  // namespace mi355

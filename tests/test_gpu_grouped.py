@@ -1,0 +1,140 @@
+"""GPU parity of the routing tables and the grouped (per-expert) block-FP8 GEMM."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ref as tr
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _align(topk_ids, topk_weights, E):
+    from lightllm_amd.fused_moe import moe_align_fused
+
+    P = topk_ids.numel()
+    idx = torch.full((E, P), -7, dtype=torch.int32, device="cuda")
+    w = torch.full((E, P), -7.0, dtype=torch.float32, device="cuda")
+    cnt = torch.empty((E,), dtype=torch.int32, device="cuda")
+    moe_align_fused(idx, w, cnt, topk_ids.cuda(), topk_weights.cuda())
+    torch.cuda.synchronize()
+    return idx, w, cnt
+
+
+def _check_align(topk_ids, topk_weights, E):
+    """The reference test's bincount / nonzero oracle (unit_tests/common/fused_moe/test_grouped_fused_moe.py:80-112),
+    in the ordered form, plus the C oracle for the whole table."""
+    idx, w, cnt = _align(topk_ids, topk_weights, E)
+    flat = topk_ids.flatten().long()
+    assert torch.equal(cnt.cpu(), torch.bincount(flat, minlength=E).to(torch.int32))
+    o_idx, o_w, o_cnt = oracle.moe_align_fused(topk_ids.numpy(), topk_weights.numpy(), E)
+    assert np.array_equal(cnt.cpu().numpy(), o_cnt)
+    idx, w = idx.cpu().numpy(), w.cpu().numpy()
+    for e in range(E):
+        c = o_cnt[e]
+        assert np.array_equal(idx[e, :c], o_idx[e, :c])
+        assert np.array_equal(w[e, :c], o_w[e, :c])
+        assert np.all(idx[e, c:] == -7), "wrote past the expert's count"
+
+
+def test_moe_align_fused_reference_vectors(hip):
+    print("moe_align_fused", flush=True)
+    ids = torch.tensor([[0, 1, 2], [0, 3, 1], [3, 1, 4]], dtype=torch.int32)
+    w = torch.tensor([[0.3, 0.7, 0.1], [0.2, 0.8, 0.4], [0.5, 0.6, 0.9]], dtype=torch.float32)
+    _check_align(ids, w, 5)
+    ids = (torch.arange(128 * 17, dtype=torch.int32).reshape(128, 17) % 5).contiguous()
+    _check_align(ids, torch.arange(ids.numel(), dtype=torch.float32).reshape(128, 17), 5)
+    base = torch.tensor([[0, 1, 2], [0, 3, 1], [3, 1, 4], [2, 0, 4]], dtype=torch.int32)
+    ids = base.repeat(1281, 1)[:5121].contiguous()
+    _check_align(ids, torch.arange(ids.numel(), dtype=torch.float32).reshape(5121, 3), 257)
+    ids = (torch.arange(5121 * 8, dtype=torch.int32).reshape(5121, 8) % 257).contiguous()
+    _check_align(ids, torch.arange(ids.numel(), dtype=torch.float32).reshape(5121, 8), 257)
+
+
+def test_moe_align2_reference_vectors(hip):
+    """Golden vectors of the reference's test_moe_align2 (test_grouped_fused_moe.py:219-258)."""
+    from lightllm_amd.fused_moe import moe_align2
+
+    print("moe_align2", flush=True)
+    cnt = torch.tensor([8, 0, 60, 16], dtype=torch.int32, device="cuda")
+    t = moe_align2(100, cnt, block_m=16).cpu()
+    assert t.shape[0] == min(100, -(-(100 + 4 * 15) // 16))
+    assert t[:, 0].tolist() == [0, 2, 2, 2, 2, 3, -1, -1, -1, -1]
+    assert t[:6, 1].tolist() == [0, 0, 1, 2, 3, 0]
+    assert t[:6, 2].tolist() == [0, 8, 24, 40, 56, 68]
+    cnt = torch.zeros((10,), dtype=torch.int32, device="cuda")
+    cnt[0] = 8
+    t = moe_align2(8, cnt, block_m=16).cpu()
+    assert t.shape[0] == 8 and t[0, 0] == 0 and bool((t[1:, 0] == -1).all())
+
+
+def _grouped_case(T, E, topk, N, K, block_m, mul_w, seed):
+    from lightllm_amd.fused_moe import grouped_matmul, moe_align2
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    ids, tw = H.routing(T, E, topk, seed=seed)
+    idx, w, cnt = _align(ids, tw, E)
+    x = H.activations(T, K, seed=seed + 1).cuda()
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, -(-N // 128), K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=seed + 10 + e, device="cuda")
+    P = T * topk
+    out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=mul_w, use_fp8_w8a8=True,
+                   run_config={"BLOCK_SIZE_M": block_m} if block_m else None)
+    torch.cuda.synchronize()
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    ref_bits = oracle.grouped_block_gemm(tr.bits_of(xq), xs.cpu().numpy(), tr.bits_of(wq), ws.cpu().numpy(),
+                                         idx.cpu().numpy(), w.cpu().numpy(), cnt.cpu().numpy(), topk, mul_w)
+    ref = tr.bf16_from_bits(ref_bits).float()
+    got = out.float().cpu()
+    assert not torch.isnan(got).any(), "a routed row was not written"
+    cos, rel = H.gemm_metrics(got, ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+    assert (got - ref).abs().max() <= ref.abs().max() * 2 ** -7
+
+
+@pytest.mark.parametrize("block_m", [None, 16, 32, 64, 128])
+@pytest.mark.parametrize("mul_w,topk", [(False, 4), (True, 1)])
+def test_grouped_vs_oracle(hip, block_m, mul_w, topk):
+    print(f"grouped block_m={block_m} mul_w={mul_w} topk={topk}", flush=True)
+    _grouped_case(T=96 if topk > 1 else 300, E=12, topk=topk, N=384, K=512, block_m=block_m, mul_w=mul_w, seed=70)
+
+
+def test_grouped_empty_and_single_token_experts(hip):
+    """More experts than tokens: most experts get no rows, some one row; N tail (200 % 128 != 0)."""
+    print("grouped sparse experts", flush=True)
+    _grouped_case(T=5, E=40, topk=2, N=200, K=256, block_m=None, mul_w=False, seed=80)
+
+
+def test_grouped_deepseek_shape_sampled(hip):
+    """The routed-expert config at a reduced expert count (16 of 256 experts, same N/K, Zipf routing):
+    every routed row is checked against the torch fp32 dequant-matmul of its expert."""
+    from lightllm_amd.fused_moe import grouped_matmul
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print("grouped dsv3-shaped", flush=True)
+    T, E, topk, N, K = 1024, 16, 8, 4096, 7168
+    ids, tw = H.routing(T, E, topk, seed=90)
+    idx, w, cnt = _align(ids, tw, E)
+    x = H.activations(T, K, seed=91).cuda()
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, N // 128, K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=100 + e, device="cuda")
+    P = T * topk
+    out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=False, use_fp8_w8a8=True)
+    torch.cuda.synchronize()
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    dx = tr.dequant(xq, xs, 1, 128)
+    pair_expert = ids.flatten().cuda().long()
+    for e in range(E):
+        rows = torch.nonzero(pair_expert == e).flatten()
+        if rows.numel() == 0:
+            continue
+        ref = dx[rows // topk] @ tr.dequant(wq[e], ws[e], 128, 128).T
+        cos, rel = H.gemm_metrics(out[rows].float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (e, cos, rel)

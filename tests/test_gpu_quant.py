@@ -1,0 +1,127 @@
+"""GPU parity of per_token_group_quant_fp8 against the CPU oracle: bytes and scale bits must be identical."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ref as tr
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(x: torch.Tensor, **kw):
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    xq, xs = per_token_group_quant_fp8(x.cuda(), 128, **kw)
+    torch.cuda.synchronize()
+    return xq, xs
+
+
+def _check(x: torch.Tensor, xq, xs):
+    q_ref, s_ref = oracle.group_quant_fp8(tr.bits_of(x))
+    q = tr.bits_of(xq)
+    s = tr.bits_of(xs.contiguous())
+    nq = int((q != q_ref).sum())
+    ns = int((s != s_ref.view(np.uint32)).sum())
+    assert ns == 0, f"{ns} scale words differ"
+    assert nq == 0, f"{nq} of {q.size} fp8 bytes differ"
+
+
+@pytest.mark.parametrize("M,K", [(1, 128), (1, 4096), (8, 4096), (32, 4096), (64, 14336), (257, 7168), (33, 384), (4096, 2048)])
+def test_bit_exact_normal(hip, M, K):
+    print(f"quant M={M} K={K}", flush=True)
+    x = H.activations(M, K, seed=M * 131 + K)
+    _check(x, *_run(x))
+
+
+def test_bit_exact_outliers_zero_row(hip):
+    print("quant outliers 2048x7168", flush=True)
+    x = H.activations(2048, 7168, seed=4, outliers=True, zero_row=True)
+    xq, xs = _run(x)
+    _check(x, xq, xs)
+    # the all-zero row: eps floor -> scale bits of fp32(1e-10)/448, all bytes zero
+    assert np.all(tr.bits_of(xs[0].contiguous()) == 0x2A7B5123)
+    assert np.all(tr.bits_of(xq[0].contiguous()) == 0)
+
+
+def test_wide_dynamic_range(hip):
+    """Groups whose magnitudes span the whole bf16 range, including subnormal inputs and values below eps."""
+    print("quant dynamic range", flush=True)
+    g = H.gen(7)
+    M, K = 512, 1024
+    expo = torch.randint(-140, 120, (M, K // 128, 1), generator=g).float()
+    x = (torch.randn((M, K // 128, 128), generator=g) * torch.exp2(expo)).reshape(M, K).to(torch.bfloat16)
+    _check(x, *_run(x))
+
+
+def test_every_bf16_value(hip):
+    """Every finite bf16 pattern as an element, against several group maxima."""
+    print("quant all bf16 patterns", flush=True)
+    bits = np.arange(65536, dtype=np.uint16)
+    finite = bits[(bits & 0x7F80) != 0x7F80]
+    vals = tr.bf16_from_bits(finite)  # 65280 values
+    n = vals.numel() // 127 * 127
+    rows = []
+    for top in [448.0, 1.0, 3.0e38, 1e-3, 7.25, 1e-20]:
+        body = vals[:n].reshape(-1, 127).clone()
+        body = torch.where(body.abs().float() <= top, body, torch.zeros_like(body))
+        lead = torch.full((body.shape[0], 1), top, dtype=torch.bfloat16)
+        rows.append(torch.cat([lead, body], dim=1))
+    x = torch.cat(rows, dim=0).contiguous()
+    _check(x, *_run(x))
+
+
+def test_column_major_scales(hip):
+    print("quant column-major scales", flush=True)
+    x = H.activations(130, 1024, seed=9)
+    xq, xs = _run(x, column_major_scales=True, scale_tma_aligned=True)
+    assert xs.shape == (130, 8) and xs.stride() == (1, 132)
+    _check(x, xq, xs)
+
+
+def test_into_caller_buffers(hip):
+    from lightllm_amd.quantization import lightllm_per_token_group_quant_fp8
+
+    x = H.activations(48, 512, seed=11).cuda()
+    xq = torch.empty_like(x, dtype=torch.float8_e4m3fn)
+    xs = torch.empty((4, 48), dtype=torch.float32, device="cuda").t()  # column-major view
+    assert lightllm_per_token_group_quant_fp8(x, 128, xq, xs) is None
+    torch.cuda.synchronize()
+    _check(x.cpu(), xq, xs)
+
+
+def test_full_size_properties(hip):
+    """The bandwidth config [16384,7168] with outliers and a zero row: bit-exact on a row sample, and
+    size-independent properties on the whole tensor."""
+    print("quant full size 16384x7168", flush=True)
+    x = H.activations(16384, 7168, seed=0, outliers=True, zero_row=True)
+    xq, xs = _run(x)
+    rows = np.r_[0:64, 8000:8064, 16320:16384]
+    q_ref, s_ref = oracle.group_quant_fp8(tr.bits_of(x)[rows])
+    assert np.array_equal(tr.bits_of(xq)[rows], q_ref)
+    assert np.array_equal(tr.bits_of(xs.contiguous())[rows], s_ref.view(np.uint32))
+    qb = xq.view(torch.uint8)
+    assert int(((qb & 0x7F) == 0x7F).sum()) == 0, "NaN code produced"
+    # every non-zero group holds its maximum as +-448
+    top = (qb & 0x7F).view(16384, 56, 128).amax(dim=-1)
+    nonzero = x.cuda().view(16384, 56, 128).abs().amax(dim=-1) > 1e-10
+    assert bool((top[nonzero] == 0x7E).all())
+    # signs survive
+    sign_in = x.cuda().view(torch.int16) < 0
+    sign_out = (qb & 0x80) != 0
+    assert bool((sign_out == sign_in).all())
+    # the scale is the group amax over 448 (IEEE division, evaluated by torch on the CPU)
+    amax = x.float().view(16384, 56, 128).abs().amax(dim=-1).clamp_min(1e-10)
+    assert torch.equal(xs.cpu(), amax / 448.0)
+
+
+def test_preconditions(hip):
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    with pytest.raises(AssertionError):
+        per_token_group_quant_fp8(torch.zeros((4, 100), dtype=torch.bfloat16, device="cuda"), 128)
+    with pytest.raises(AssertionError):
+        per_token_group_quant_fp8(torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")[:, ::2], 64)
+    xq, xs = per_token_group_quant_fp8(torch.zeros((0, 256), dtype=torch.bfloat16, device="cuda"), 128)
+    assert xq.shape == (0, 256) and xs.shape == (0, 2)
