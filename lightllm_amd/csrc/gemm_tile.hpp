@@ -80,7 +80,7 @@ struct TileCfg {
     static constexpr int kScaleOff = NSTAGE * kStage;
     static constexpr int kWsOff = kScaleOff + NSTAGE * BM * 4;  // weight scales of the whole K range
     static constexpr int NBC = BN >= 128 ? BN / 128 : 1;        // 128-wide scale blocks a tile spans
-    static constexpr int lds_bytes(int KB) { return kWsOff + NBC * KB * 4; }
+    static constexpr int lds_bytes(int KB) { return kWsOff + NBC * KB * 4 + 16; }  // + the split-K arrival word
     static_assert(XG % kWaves == 0 || kWaves % XG == 0, "X tile rows must split over the waves");
     static_assert(WG % kWaves == 0 || kWaves % WG == 0, "W tile rows must split over the waves");
     static_assert(WNS <= 128 && 128 % WNS == 0, "a wave's n span must sit inside one 128-wide scale block");
@@ -304,10 +304,12 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             for (int j = 0; j < TN; ++j) *(v4f *)(mine + ((i * TN + j) * Cfg::kThreads + tid) * 4) = acc[i][j];
         __threadfence();
         __syncthreads();
-        __shared__ uint32_t arrived;
-        if (tid == 0) arrived = atomicAdd(p.counters + tile_id, 1u);
+        // (kept in the dynamic allocation: a static __shared__ object would push static + opt-in dynamic
+        // LDS past the 160 KiB a workgroup may ask for)
+        volatile uint32_t *arrived = (volatile uint32_t *)(lds + Cfg::kWsOff + Cfg::NBC * KB * 4);
+        if (tid == 0) *arrived = atomicAdd(p.counters + tile_id, 1u);
         __syncthreads();
-        if (arrived != (uint32_t)p.splits - 1u) return;
+        if (*arrived != (uint32_t)p.splits - 1u) return;
         __threadfence();
         const float *base = p.partials + (int64_t)tile_id * p.splits * kTileElems;
 #pragma unroll

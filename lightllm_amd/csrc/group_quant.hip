@@ -17,7 +17,8 @@
 //     the CPU); for any other eps the kernel takes a true division.
 //   * x/s is formed as y0 = x*r, y = fma(fma(-y0,s,x), r, y0) with r = RN(1/s) (a true division,
 //     once per lane).  For every pair (bf16 amax, bf16 |x| <= amax) this equals RN(x/s) whenever
-//     |x/s| >= 2^-10, and below that both round to the e4m3 zero - also checked exhaustively on the CPU.
+//     |x/s| >= 2^-10, and below that both round to the e4m3 zero - also checked exhaustively on the CPU
+//     (oracle_fast_quant_mismatches in the test oracle replays exactly these operations).
 #include "common.hpp"
 
 namespace mi355 {
@@ -44,13 +45,16 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// RN(x/s) wherever it matters (see the header), with the sign taken from x: the correction step turns
+// -0 into +0, and the reference's -0/s = -0 keeps its sign bit through the cast (byte 0x80).
+// No clamp is needed: |x| <= amax and s = RN(max(amax,eps)/448) bound |x/s| by 448*(1+2^-23), which the
+// e4m3 cast rounds to 448, exactly what clamp-then-cast gives.
 __device__ __forceinline__ float quot(float x, float s, float r) {
     float y0 = x * r;
     float e = __builtin_fmaf(-y0, s, x);
-    return __builtin_fmaf(e, r, y0);
+    float y = __builtin_fmaf(e, r, y0);
+    return as_f32((as_u32(y) & 0x7fffffffu) | (as_u32(x) & 0x80000000u));
 }
-
-__device__ __forceinline__ float clamp448(float y) { return __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f); }
 
 // Quantize one 16-byte chunk; the group amax is shared through the DPP row.
 __device__ __forceinline__ void quant_chunk(const v4i &v, float eps, bool eps_is_default, v2i &out, float &scale) {
@@ -78,7 +82,7 @@ __device__ __forceinline__ void quant_chunk(const v4i &v, float eps, bool eps_is
     f[4] = as_f32(d2 << 16); f[5] = as_f32(d2 & 0xffff0000u);
     f[6] = as_f32(d3 << 16); f[7] = as_f32(d3 & 0xffff0000u);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = clamp448(quot(f[i], s, r));
+    for (int i = 0; i < 8; ++i) f[i] = quot(f[i], s, r);
     int w0 = 0, w1 = 0;
     w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], w0, false);
     w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);

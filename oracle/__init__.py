@@ -40,6 +40,8 @@ def lib() -> ctypes.CDLL:
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.oracle_moe_align2_rows.restype = ctypes.c_int64
         _lib.oracle_moe_align2_rows.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+        _lib.oracle_fast_quant_mismatches.restype = ctypes.c_int64
+        _lib.oracle_fast_quant_mismatches.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32]
     return _lib
 
 
@@ -176,6 +178,11 @@ def grouped_block_gemm(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weights, 
         I64(N), I64(K), I32(bn), I32(bk), I32(1 if mul_routed_weight else 0), _p(out),
     )
     return out
+
+
+def fast_quant_mismatches(amax_lo: int = 0, amax_hi: int = 0x7F80, step: int = 1) -> int:
+    """Pairs (bf16 amax, bf16 x) for which the HIP quantizer's division shortcut would differ from IEEE."""
+    return int(lib().oracle_fast_quant_mismatches(amax_lo, amax_hi, step))
 
 
 def silu_and_mul(x_bf16_bits) -> np.ndarray:

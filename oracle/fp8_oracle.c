@@ -355,6 +355,54 @@ void oracle_moe_sum_reduce(const uint16_t *in, int64_t T, int32_t topk, int64_t 
         }
 }
 
+/*
+ * Replays, on the CPU, the exact operation sequence the HIP quantizer uses in place of two IEEE
+ * divisions (csrc/group_quant.hip: quant_chunk/quot), for every bf16 group maximum with bit pattern in
+ * [amax_lo, amax_hi) stepping by `step`, against every bf16 element of either sign with |x| <= amax
+ * (and every |x| < eps when the eps floor applies).  Returns how many (amax, x) pairs give a byte or a
+ * scale different from the IEEE closed form above.  Zero for the whole range means the kernel's
+ * shortcut is exact; it must stay in step with the kernel source.
+ */
+int64_t oracle_fast_quant_mismatches(uint32_t amax_lo, uint32_t amax_hi, uint32_t step) {
+    const float eps = 1e-10f, c448 = 1.0f / 448.0f;
+    int64_t bad = 0;
+    for (uint32_t ab = amax_lo; ab < amax_hi && ab <= 0x7f7fu; ab += step) {
+        float amax = oracle_bf16_to_f32((uint16_t)ab);
+        uint32_t xmax = ab;
+        if (!(amax > eps)) {
+            if (ab != 0) continue;       /* every maximum below eps gives the same scale: test it once, */
+            amax = eps;
+            xmax = 0x2edbu;              /* against every bf16 magnitude below 1e-10 */
+        }
+        volatile float s_ref = amax / 448.0f;
+        /* kernel: scale */
+        float q0 = amax * c448;
+        float s = fmaf(fmaf(-q0, 448.0f, amax), c448, q0);
+        if (f32_to_bits(s) != f32_to_bits(s_ref)) { ++bad; continue; }
+        volatile float r = 1.0f / s;
+        for (uint32_t xb = 0; xb <= xmax; ++xb) {
+            for (uint32_t sign = 0; sign <= 0x8000u; sign += 0x8000u) {
+                float x = oracle_bf16_to_f32((uint16_t)(xb | sign));
+                /* reference */
+                volatile float y = x / s_ref;
+                float cl = y;
+                if (cl > 448.0f) cl = 448.0f;
+                if (cl < -448.0f) cl = -448.0f;
+                uint8_t want = oracle_f32_to_e4m3fn(cl);
+                /* kernel */
+                float y0 = x * r;
+                float e = fmaf(-y0, s, x);
+                float y1 = fmaf(e, r, y0);
+                float fixed = bits_to_f32((f32_to_bits(y1) & 0x7fffffffu) | (f32_to_bits(x) & 0x80000000u));
+                uint8_t got = oracle_f32_to_e4m3fn(fixed);
+                if ((got & 0x7f) == 0x7f) got = (uint8_t)((got & 0x80) | 0x7e); /* the hardware cast saturates */
+                if (got != want) ++bad;
+            }
+        }
+    }
+    return bad;
+}
+
 /* Bulk helpers so tests can sweep millions of values without a Python loop. */
 void oracle_f32_to_e4m3fn_array(const float *x, int64_t n, uint8_t *out) {
     for (int64_t i = 0; i < n; ++i) out[i] = oracle_f32_to_e4m3fn(x[i]);
