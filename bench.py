@@ -1,0 +1,304 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-FP8 W8A8 linear path on one MI355X.
+
+One "step" is one pass of the path over one batch of synthetic input: per_token_group_quant_fp8 of the
+bf16 activations followed by w8a8_block_fp8_matmul against block-quantized weights, everything resident
+in HBM.  The headline workload is the DeepSeek-V3-shaped prefill gate_up linear (M=4096, N=36864, K=7168),
+the configuration the FP8-MFMA target is stated on; the other shapes of the benchmark plan (decode-size M,
+the standalone quantizer, the routed-expert grouped GEMM) are timed too and reported under "others".
+
+Prints ONE JSON line.  Runs on one GPU only.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP8_MFMA_PEAK_TFLOPS = 5033.0  # 256 CU x 4 SIMD x 2048 flop/clk x 2.4 GHz, dense
+HBM_PEAK_GBS = 8000.0
+
+
+def _events(n):
+    import torch
+
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def _time_calls(fn, iters, warm):
+    """Average duration of `fn` in microseconds, HIP events on torch's current stream (the launch stream)."""
+    import torch
+
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    s, e = _events(2)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) * 1e3 / iters
+
+
+def gemm_bytes(M, N, K):
+    return M * K + N * K + 2 * M * N + 4 * M * (K // 128) + 4 * ((N + 127) // 128) * (K // 128)
+
+
+def quant_bytes(M, K):
+    return M * K * 3 + 4 * M * (K // 128)
+
+
+def make_weight(N, K, seed, device):
+    """~N(0, 0.02) bf16 weight, block-quantized by the library's own load-time quantizer."""
+    import torch
+
+    from lightllm_amd.quantization import mm_weight_quant
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    w = (torch.randn((N, K), generator=g, device=device, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    q, s = mm_weight_quant(w)
+    return q, s
+
+
+def make_act(M, K, seed, device, outliers=False):
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn((M, K), generator=g, device=device, dtype=torch.float32)
+    if outliers:
+        x = torch.where(torch.rand((M, K), generator=g, device=device) < 0.01, x * 50.0, x)
+        x[0] = 0.0
+    return x.to(torch.bfloat16)
+
+
+def cpu_baseline(M_sample, N, K):
+    """The reference's torch dequant+matmul form in fp32 plus its CPU quantizer, timed on the host cores
+    on a row sample of the headline workload (full N and K, M_sample of the 4096 rows)."""
+    import torch
+
+    from oracle import torch_ref as tr
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((M_sample, K), generator=g).to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g) * 0.02).to(torch.bfloat16)
+    wq, ws = tr.block_weight_quant(w)
+    del w
+
+    def step():
+        xq, xs = tr.group_quant(x)
+        return tr.dequant_matmul(xq, xs, wq, ws)
+
+    step()
+    times = []
+    t_end = time.perf_counter() + 20.0
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": round(2.0 * M_sample * N * K / med / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"rows 0..{M_sample - 1} of the M=4096 activations, full N={N} K={K}; torch CPU fp32 "
+                  f"quant + dequant + matmul, median of {len(times)} runs ({med:.2f} s each), os.cpu_count()={os.cpu_count()}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|grouped (for profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the path; this build has no multi-GPU leg (--gpus must be 1)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from lightllm_amd import _lib
+    from lightllm_amd.fused_moe import grouped_matmul, moe_align_fused
+    from lightllm_amd.quantization import (lightllm_per_token_group_quant_fp8, per_token_group_quant_fp8,
+                                           w8a8_block_fp8_matmul)
+
+    _lib.lib()  # fail loudly if the HIP library is not built
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    info = _lib.device_info()
+    derived_peak = info["compute_units"] * 4 * 2048 * info["clock_khz"] * 1e3 / 1e12
+
+    M, N, K = 4096, 36864, 7168
+    run_all = args.only is None
+    result = {}
+    others = []
+
+    if run_all or args.only == "headline":
+        x = make_act(M, K, 0, dev)
+        wq, ws = make_weight(N, K, 1, dev)
+        xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=dev)
+        xs = torch.empty((M, K // 128), dtype=torch.float32, device=dev)
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        wq_t, ws_t = wq.t(), ws.t()
+
+        def step():
+            lightllm_per_token_group_quant_fp8(x, 128, xq, xs)
+            w8a8_block_fp8_matmul(xq, wq_t, xs, ws_t, out, [128, 128], dtype=torch.bfloat16)
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev = _events(2 * args.steps)
+        for i in range(args.steps):
+            lightllm_per_token_group_quant_fp8(x, 128, xq, xs)
+            ev[2 * i].record()          # brackets only the GEMM kernel, on the stream it is launched on
+            w8a8_block_fp8_matmul(xq, wq_t, xs, ws_t, out, [128, 128], dtype=torch.bfloat16)
+            ev[2 * i + 1].record()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        ms_per_step = elapsed * 1e3 / args.steps
+        gemm_us = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) * 1e3 / args.steps
+        flops = 2.0 * M * N * K
+        value = flops / (ms_per_step * 1e-3) / 1e12
+        achieved = flops / (gemm_us * 1e-6) / 1e12
+        result = {
+            "metric": "block-FP8 GEMM TFLOP/s (% FP8 MFMA peak); quant GB/s (% HBM peak), 1 GPU",
+            "value": round(value, 1),
+            "unit": "TFLOP/s",
+            "n_gpus": 1,
+            "steps": args.steps,
+            "warmup": args.warmup,
+            "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": True,
+            "scaling": "weak",
+            "vs_baseline": None,
+            "dtype": "fp8_e4m3 x fp8_e4m3 -> f32 accumulate -> bf16",
+            "data": "synthetic (seeded N(0,1) bf16 activations; N(0,0.02) weights block-quantized 128x128)",
+            "config": {
+                "workload": "DeepSeek-V3-shaped prefill gate_up linear: per_token_group_quant_fp8([4096,7168] bf16) "
+                            "+ w8a8_block_fp8_matmul(M=4096, N=36864, K=7168), bf16 out",
+                "M": M, "N": N, "K": K, "block": [128, 128],
+            },
+            "roofline": {
+                "bound": "mfma",
+                "kernel": "block_fp8_gemm_tile_kernel<256,256,2,4,2,dense>",
+                "achieved": round(achieved, 1),
+                "peak": FP8_MFMA_PEAK_TFLOPS,
+                "unit": "TFLOP/s",
+                "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
+                "traffic": None,
+                "launch_us": round(gemm_us, 2),
+                "algorithmic_flops_per_launch": flops,
+                "peak_derived_from_device": round(derived_peak, 1),
+            },
+        }
+        del x, wq, ws, xq, xs, out, wq_t, ws_t
+        torch.cuda.empty_cache()
+
+    if (run_all and not args.no_others) or args.only == "quant":
+        # standalone quantizer bandwidth test: [16384,7168] with 1% x50 outliers and an all-zero row
+        Mq, Kq = 16384, 7168
+        x = make_act(Mq, Kq, 4, dev, outliers=True)
+        xq = torch.empty((Mq, Kq), dtype=torch.float8_e4m3fn, device=dev)
+        xs = torch.empty((Mq, Kq // 128), dtype=torch.float32, device=dev)
+        us = _time_calls(lambda: lightllm_per_token_group_quant_fp8(x, 128, xq, xs), 50, 5)
+        gbs = quant_bytes(Mq, Kq) / us / 1e3
+        others.append({"name": "per_token_group_quant_fp8 [16384,7168]", "us": round(us, 2), "GB/s": round(gbs, 1),
+                       "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
+        del x, xq, xs
+        torch.cuda.empty_cache()
+
+    if (run_all and not args.no_others) or args.only == "decode":
+        # Llama-3-8B decode linears; weights rotate through 5 copies so that no launch finds them in the
+        # 256 MB memory-side cache
+        for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down")]:
+            copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(5)]
+            for Md in (1, 8, 32, 64):
+                xq, xs = per_token_group_quant_fp8(make_act(Md, Kd, 20 + Md, dev), 128)
+                out = torch.empty((Md, Nd), dtype=torch.bfloat16, device=dev)
+                idx = [0]
+
+                def call():
+                    q, s = copies[idx[0] % 5]
+                    idx[0] += 1
+                    w8a8_block_fp8_matmul(xq, q.t(), xs, s.t(), out, [128, 128])
+
+                us = _time_calls(call, 40, 10)
+                gbs = gemm_bytes(Md, Nd, Kd) / us / 1e3
+                others.append({"name": f"llama3-8b {name} M={Md} N={Nd} K={Kd}", "us": round(us, 2),
+                               "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                               "TFLOP/s": round(2.0 * Md * Nd * Kd / us / 1e6, 2)})
+            del copies
+            torch.cuda.empty_cache()
+
+    if (run_all and not args.no_others) or args.only == "prefill":
+        for (Np, Kp, name) in [(7168, 18432, "down"), (2112, 7168, "q_a+kv_a")]:
+            wq, ws = make_weight(Np, Kp, 30, dev)
+            xq, xs = per_token_group_quant_fp8(make_act(M, Kp, 31, dev), 128)
+            out = torch.empty((M, Np), dtype=torch.bfloat16, device=dev)
+            us = _time_calls(lambda: w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128]), 20, 5)
+            tf = 2.0 * M * Np * Kp / us / 1e6
+            others.append({"name": f"deepseek-v3 {name} M=4096 N={Np} K={Kp}", "us": round(us, 2),
+                           "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / FP8_MFMA_PEAK_TFLOPS, 4)})
+            del wq, ws, xq, xs, out
+            torch.cuda.empty_cache()
+
+    if (run_all and not args.no_others) or args.only == "grouped":
+        # routed experts: 4096 tokens x top-8 over 256 experts, Zipf(1.1) popularity; weights are random fp8
+        # bytes here (11.3 GB; values do not change the timing), scales uniform in [0.5, 1.5) * 2e-4
+        T, E, topk = 4096, 256, 8
+        g = torch.Generator(device=dev).manual_seed(5)
+        perm = torch.randperm(E, generator=g, device=dev)
+        p = torch.zeros(E, device=dev)
+        p[perm] = 1.0 / torch.arange(1, E + 1, device=dev, dtype=torch.float32) ** 1.1
+        ids = torch.multinomial((p / p.sum()).expand(T, E), topk, replacement=False, generator=g).to(torch.int32)
+        tw = torch.softmax(torch.randn((T, topk), generator=g, device=dev), dim=-1)
+        P = T * topk
+        e2t = torch.empty((E, P), dtype=torch.int32, device=dev)
+        e2w = torch.empty((E, P), dtype=torch.float32, device=dev)
+        cnt = torch.empty((E,), dtype=torch.int32, device=dev)
+        moe_align_fused(e2t, e2w, cnt, ids, tw)
+        experts_hit = int((cnt > 0).sum())
+
+        def rand_fp8(shape):
+            b = torch.randint(0, 256, shape, dtype=torch.uint8, device=dev, generator=g)
+            return (b & 0xB7).view(torch.float8_e4m3fn)  # clears one exponent and one mantissa bit: no NaN codes
+
+        for (Ng, Kg, tk, mulw, name) in [(4096, 7168, topk, False, "gate_up"), (7168, 2048, 1, True, "down")]:
+            w = rand_fp8((E, Ng, Kg))
+            wscale = (torch.rand((E, Ng // 128, Kg // 128), generator=g, device=dev) + 0.5) * 2e-4
+            rows = T if tk == topk else P
+            xq, xs = per_token_group_quant_fp8(make_act(rows, Kg, 40, dev), 128)
+            out = torch.empty((P, Ng), dtype=torch.bfloat16, device=dev)
+            us = _time_calls(lambda: grouped_matmul(P, xq, xs, cnt, e2t, e2w, w, wscale, tk, out, mulw, True), 10, 3)
+            flops = 2.0 * P * Ng * Kg
+            byts = experts_hit * Ng * Kg + rows * Kg + 2 * P * Ng
+            others.append({"name": f"deepseek-v3 routed experts {name}: {P} rows, E={E}, N={Ng} K={Kg}",
+                           "us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1), "GB/s": round(byts / us / 1e3, 1),
+                           "roofline_us": round(max(byts / HBM_PEAK_GBS / 1e3, flops / FP8_MFMA_PEAK_TFLOPS / 1e6), 1),
+                           "experts_hit": experts_hit})
+            del w, wscale, xq, xs, out
+            torch.cuda.empty_cache()
+
+    if not result:
+        result = {"metric": "partial run (--only)", "n_gpus": 1}
+    if others:
+        result["others"] = others
+    if run_all and not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(64, N, K)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,152 @@
+"""CPU checks of the drop-in boundary: the library loads and exports every symbol the header declares, the
+ctypes table covers the header, the Python functions keep the reference's signatures, and argument checks
+fire before any launch."""
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "mi355_fp8.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    names = _header_symbols()
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names, "ctypes table and header disagree"
+
+
+def test_error_strings():
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.mi355_error_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert lib.mi355_error_string(code) not in (b"ok", b"unknown error code")
+    assert lib.mi355_error_string(-99) == b"unknown error code"
+
+
+def test_pure_host_entry_points():
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    # rows of the schedule table: min(pairs, ceil((pairs + E*(bm-1))/bm))   (reference test_moe_align2)
+    assert lib.mi355_moe_align2_rows(100, 4, 16) == 10
+    assert lib.mi355_moe_align2_rows(8, 10, 16) == 8
+    assert lib.mi355_grouped_block_m(32768, 256, 4096, 7168) in (16, 32, 64, 128)
+    assert lib.mi355_block_fp8_gemm_workspace_bytes(4096, 4096, 4096, 0) == 0     # large M: no split-K
+    assert lib.mi355_block_fp8_gemm_workspace_bytes(8, 4096, 14336, 0) > 65536
+
+
+def test_preconditions_are_checked_before_launch():
+    """Null pointers and bad shapes are rejected on the host; nothing reaches the (absent) GPU."""
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.mi355_group_quant_fp8(None, None, None, 4, 100, 128, 1e-10, 1, 1, None) == -2   # K % 128
+    assert lib.mi355_group_quant_fp8(None, None, None, 4, 256, 64, 1e-10, 4, 1, None) == -6    # group != 128
+    assert lib.mi355_group_quant_fp8(None, None, None, 4, 256, 128, 1e-10, 2, 1, None) == -1   # null
+    assert lib.mi355_group_quant_fp8(None, None, None, 0, 256, 128, 1e-10, 2, 1, None) == 0    # empty
+    assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 64, 128,
+                                    None, 0, 0, None) == -6
+    assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 128, 128,
+                                    None, 0, 0, None) == -1
+    assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 0, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 128, 128,
+                                    None, 0, 0, None) == 0
+    assert lib.mi355_block_weight_quant_fp8(None, 7, None, None, 4, 4, 128, None) == -1
+    assert lib.mi355_moe_align2(None, 0, 16, 4, None, None) == -1
+
+
+REFERENCE_SIGNATURES = {
+    # (module, function): signature string of the reference's function of the same name
+    ("lightllm_amd.quantization.fp8act_quant_kernel", "per_token_group_quant_fp8"):
+        "(x, group_size, eps=1e-10, dtype=torch.float8_e4m3fn, column_major_scales=False, scale_tma_aligned=False, alloc_func=torch.empty)",
+    ("lightllm_amd.quantization.fp8act_quant_kernel", "lightllm_per_token_group_quant_fp8"):
+        "(x, group_size, x_q, x_s, eps=1e-10, dtype=torch.float8_e4m3fn)",
+    ("lightllm_amd.quantization.fp8w8a8_block_gemm_kernel", "w8a8_block_fp8_matmul"):
+        "(A, B, Ascale, Bscale, C, block_size, dtype=torch.bfloat16, run_config=None)",
+    ("lightllm_amd.quantization.fp8w8a8_block_quant_kernel", "weight_quant"): "(x, block_size=128)",
+    ("lightllm_amd.quantization.fp8w8a8_block_quant_kernel", "mm_weight_quant"): "(x, block_size=128)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "moe_align_fused"):
+        "(expert_to_token_index, expert_to_weight, expert_token_num, topk_ids, topk_weights)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "moe_align2"): "(token_num_mul_topk_num, exports_token_num, block_m)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "grouped_matmul"):
+        "(token_num_mul_topk_num, token_inputs, token_input_scale, expert_to_token_num, expert_to_token_index, "
+        "expert_to_weights, expert_weights, expert_to_weights_scale, topk_num, out, mul_routed_weight, use_fp8_w8a8, "
+        "alloc_tensor_func=torch.empty, reused_mblock_infos=None, run_config=None, bias=None)",
+}
+
+
+def _sig_string(fn):
+    parts = []
+    for p in inspect.signature(fn).parameters.values():
+        if p.default is inspect._empty:
+            parts.append(p.name)
+        else:
+            d = p.default
+            if d is torch.empty:
+                d = "torch.empty"
+            elif isinstance(d, torch.dtype):
+                d = str(d)
+            parts.append(f"{p.name}={d}")
+    return "(" + ", ".join(parts) + ")"
+
+
+@pytest.mark.parametrize("key", sorted(REFERENCE_SIGNATURES))
+def test_python_signatures_match_the_reference(key):
+    import importlib
+
+    mod, name = key
+    fn = getattr(importlib.import_module(mod), name)
+    assert _sig_string(fn) == REFERENCE_SIGNATURES[key]
+
+
+def test_quantization_method_surface():
+    """The plug-in object exposes what LightLLM's MMWeightTpl calls (quantize_method.py:25-149, w8a8.py:418-533)."""
+    from lightllm_amd.quantization import QUANTMETHODS, QuantizationMethod, WeightPack
+
+    cls = QUANTMETHODS._quant_methods["fp8w8a8-b128"]["cuda"]
+    assert issubclass(cls, QuantizationMethod)
+    assert QUANTMETHODS._quant_methods["fp8w8a8-b128-triton"]["cuda"] is cls
+    with pytest.raises(ValueError):
+        QUANTMETHODS.get("no-such-method")
+    with pytest.raises(ValueError):
+        QUANTMETHODS.get("fp8w8a8-b128", platform="musa")
+    apply_sig = list(inspect.signature(cls.apply).parameters)
+    assert apply_sig == ["self", "input_tensor", "weight_pack", "out", "workspace", "use_custom_tensor_mananger", "bias"]
+    for meth in ("quantize", "create_weight", "create_moe_weight", "load_weight", "load_weight_scale",
+                 "load_weight_zero_point", "_create_weight", "_split_weight_pack", "_check_weight_need_quanted"):
+        assert callable(getattr(cls, meth))
+    m = cls()
+    assert m.block_size == 128 and m.weight_scale_suffix == "weight_scale_inv" and m.has_weight_scale
+    assert m.method_name.startswith("fp8w8a8-b128")
+    pack = WeightPack(weight=torch.zeros((2, 4, 4)), weight_scale=torch.ones((2, 1, 1)))
+    assert pack.load_ok == [False, False, True]
+    sub = pack.get_expert(1)
+    assert sub.weight.shape == (4, 4) and sub.weight_scale.shape == (1, 1) and sub.weight_zero_point is None
+    # fused weights are split as views along dim -2, scales in units of 128 rows
+    big = WeightPack(weight=torch.zeros((384, 256)), weight_scale=torch.zeros((3, 2)))
+    parts = m._split_weight_pack(big, [256, 128], -2, [2, 1], -2)
+    assert [p.weight.shape[0] for p in parts] == [256, 128] and [p.weight_scale.shape[0] for p in parts] == [2, 1]
+    assert parts[1].weight.data_ptr() == big.weight[256:].data_ptr()
+
+
+def test_operators_refuse_cpu_tensors():
+    """No CPU fallback: the operators raise instead of computing on the host."""
+    from lightllm_amd._lib import Mi355Error
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    with pytest.raises(Mi355Error):
+        per_token_group_quant_fp8(torch.zeros((2, 128), dtype=torch.bfloat16), 128)

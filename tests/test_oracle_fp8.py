@@ -1,0 +1,285 @@
+"""Pins the CPU oracle (oracle/fp8_oracle.c) against facts it does not itself compute:
+known-answer bytes, torch's own float8 cast, the reference's torch closed forms, special cases whose answer
+the arithmetic fixes, and brute force in float64."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import torch_ref as tr
+from tests import helpers as H
+
+
+# ---- the e4m3fn cast -------------------------------------------------------------------------------------
+KAT = [  # (value, byte): RTNE, subnormals, no saturation (measured facts about the float8_e4m3fn format)
+    (0.0, 0x00), (1.0, 0x38), (448.0, 0x7E), (449.0, 0x7E), (464.0, 0x7E), (465.0, 0x7F), (480.0, 0x7F),
+    (1000.0, 0x7F), (-1000.0, 0xFF), (2.0 ** -10, 0x00), (2.0 ** -9, 0x01), (1.5 * 2.0 ** -9, 0x02),
+    (17.0, 0x58), (18.0, 0x59), (19.0, 0x5A), (-1.0, 0xB8), (2.0 ** -6, 0x08), (0.875 * 2.0 ** -6, 0x07),
+    (240.0, 0x77), (-0.0, 0x80),
+]
+
+
+def test_e4m3_known_answers():
+    vals = np.array([v for v, _ in KAT], np.float32)
+    got = oracle.f32_to_e4m3fn(vals)
+    assert got.tolist() == [b for _, b in KAT]
+    assert oracle.f32_to_e4m3fn(np.array([np.nan], np.float32))[0] & 0x7F == 0x7F
+
+
+def test_e4m3_decode_all_codes():
+    codes = np.arange(256, dtype=np.uint8)
+    mine = oracle.e4m3fn_to_f32(codes)
+    theirs = tr.fp8_from_bits(codes).float().numpy()
+    ok = ~np.isnan(theirs)
+    assert np.array_equal(mine[ok], theirs[ok]) and np.isnan(mine[~ok]).all()
+    # every finite code survives a round trip
+    assert np.array_equal(oracle.f32_to_e4m3fn(mine[ok]), codes[ok])
+
+
+def test_e4m3_cast_matches_torch_everywhere_it_matters():
+    bits = np.arange(65536, dtype=np.uint16)
+    x = tr.bf16_from_bits(bits).float()
+    finite = ~torch.isnan(x)
+    assert np.array_equal(oracle.f32_to_e4m3fn(x.numpy())[finite.numpy()],
+                          tr.bits_of(x.to(torch.float8_e4m3fn))[finite.numpy()])
+    # dense sweep of fp32 patterns over [2^-12, 1024), both signs (every 61st pattern)
+    u = np.arange(0x39800000, 0x44800000, 61, dtype=np.uint32)
+    for sign in (0, 0x80000000):
+        f = (u | np.uint32(sign)).view(np.float32)
+        assert np.array_equal(oracle.f32_to_e4m3fn(f), tr.bits_of(torch.from_numpy(f.copy()).to(torch.float8_e4m3fn)))
+    # exact ties between neighbouring codes go to the even code
+    codes = np.arange(0, 0x7E, dtype=np.uint8)
+    lo, hi = oracle.e4m3fn_to_f32(codes), oracle.e4m3fn_to_f32(codes + 1)
+    mid = ((lo.astype(np.float64) + hi.astype(np.float64)) / 2).astype(np.float32)
+    got = oracle.f32_to_e4m3fn(mid)
+    assert np.array_equal(got, np.where(codes % 2 == 0, codes, codes + 1))
+
+
+def test_bf16_rounding_matches_torch():
+    g = H.gen(3)
+    x = torch.randn(200000, generator=g) * torch.exp2(torch.randint(-30, 30, (200000,), generator=g).float())
+    assert np.array_equal(oracle.f32_to_bf16(x.numpy()), tr.bits_of(x.to(torch.bfloat16)))
+    ties = np.array([0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001], np.uint32).view(np.float32)
+    assert oracle.f32_to_bf16(ties).tolist() == [0x3F80, 0x3F82, 0x3F80, 0x3F81]
+
+
+# ---- the activation quantizer --------------------------------------------------------------------------
+@pytest.mark.parametrize("M,K,kw", [(32, 4096, {}), (64, 1024, {"outliers": True, "zero_row": True}), (3, 128, {})])
+def test_group_quant_equals_torch_closed_form(M, K, kw):
+    x = H.activations(M, K, seed=M + K, **kw)
+    q_t, s_t = tr.group_quant(x)
+    q_c, s_c = oracle.group_quant_fp8(tr.bits_of(x))
+    assert np.array_equal(tr.bits_of(s_t), s_c.view(np.uint32))
+    assert np.array_equal(tr.bits_of(q_t), q_c)
+
+
+def test_group_quant_special_cases():
+    # all-zero group: eps floor, scale bits of fp32(1e-10)/448, bytes zero
+    z = np.zeros((1, 128), np.uint16)
+    q, s = oracle.group_quant_fp8(z)
+    assert s.view(np.uint32)[0, 0] == 0x2A7B5123 and not q.any()
+    assert np.float32(1e-10).view(np.uint32) == 0x2EDBE6FF
+    # group maximum 448 * 2^k: scale is exactly 2^k and the bytes are the exact cast of x / 2^k
+    for k in (-20, -3, 0, 5, 40):
+        vals = np.array([448.0, -448.0, 1.0, 17.0, 18.0, 19.0, 0.3125, -2.0 ** -9, 2.0 ** -10, 100.0] + [0.0] * 118,
+                        np.float32) * np.float32(2.0 ** k)
+        xb = oracle.f32_to_bf16(vals).reshape(1, 128)
+        assert np.array_equal(oracle.bf16_to_f32(xb).ravel(), vals), "test values must be bf16-exact"
+        q, s = oracle.group_quant_fp8(xb)
+        assert s[0, 0] == np.float32(2.0 ** k)
+        assert np.array_equal(q[0], oracle.f32_to_e4m3fn(vals / np.float32(2.0 ** k)))
+        assert q[0, 0] == 0x7E and q[0, 1] == 0xFE
+
+
+def test_group_quant_invariants():
+    x = H.activations(256, 2048, seed=12, outliers=True)
+    xb = tr.bits_of(x)
+    q, s = oracle.group_quant_fp8(xb)
+    xf = oracle.bf16_to_f32(xb).reshape(256, 16, 128)
+    qf = oracle.e4m3fn_to_f32(q).reshape(256, 16, 128)
+    assert not ((q & 0x7F) == 0x7F).any()                                  # never the NaN code
+    assert np.array_equal(q >> 7, xb >> 15)                                # sign bit preserved
+    # the group maximum lands on +-448
+    am = np.abs(xf).argmax(-1)
+    top = np.take_along_axis(q.reshape(256, 16, 128), am[..., None], -1)[..., 0]
+    assert np.all((top & 0x7F) == 0x7E)
+    # monotone inside a group
+    order = np.argsort(xf, axis=-1)
+    assert np.all(np.diff(np.take_along_axis(qf, order, -1), axis=-1) >= 0)
+    # rounding error of the dequantised value is at most half an e4m3 ulp of the quotient (plus fp32 slack)
+    y = xf / s[..., None]
+    ulp = np.where(np.abs(y) < 2.0 ** -6, 2.0 ** -9, 2.0 ** (np.floor(np.log2(np.maximum(np.abs(y), 1e-30))) - 3))
+    assert np.all(np.abs(qf - y) <= ulp / 2 * (1 + 1e-6))
+
+
+def test_group_quant_column_major_layout():
+    x = H.activations(10, 512, seed=13)
+    q1, s1 = oracle.group_quant_fp8(tr.bits_of(x))
+    q2, s2 = oracle.group_quant_fp8(tr.bits_of(x), column_major=True)
+    assert s2.strides == (4, 40) and np.array_equal(s1, s2) and np.array_equal(q1, q2)
+
+
+def test_kernel_division_shortcut_is_exact():
+    """The HIP quantizer replaces x/s by a multiply and two fused multiply-adds.  Replaying those operations on
+    the CPU for EVERY (bf16 group maximum, bf16 element of either sign) pair gives the IEEE bytes and scales."""
+    assert oracle.fast_quant_mismatches(0, 0x7F80, 1) == 0
+
+
+# ---- the weight quantizer ------------------------------------------------------------------------------
+@pytest.mark.parametrize("N,K", [(256, 384), (200, 300), (128, 128)])
+def test_weight_quant_equals_torch_closed_form(N, K):
+    w = H.weights(N, K, seed=N)
+    q_t, s_t = tr.block_weight_quant(w)
+    q_c, s_c = oracle.block_weight_quant(w.float().numpy())
+    assert np.array_equal(tr.bits_of(s_t), s_c.view(np.uint32))
+    assert np.array_equal(tr.bits_of(q_t), q_c)
+
+
+def test_weight_quant_quirk():
+    """Stored scale is amax/448 but the divisor is scale + 1e-6: the quotient of the block maximum stays
+    below 448 (here by about half a percent) before the cast rounds it."""
+    w = H.weights(128, 128, seed=5)
+    q, s = oracle.block_weight_quant(w.float().numpy())
+    amax = float(w.float().abs().max())
+    assert s[0, 0] == np.float32(amax) / np.float32(448.0)
+    top = np.abs(oracle.e4m3fn_to_f32(q)).max()
+    expect = amax / (float(s[0, 0]) + 1e-6)
+    assert top == oracle.e4m3fn_to_f32(oracle.f32_to_e4m3fn(np.array([expect], np.float32)))[0]
+    assert 440 < expect < 447.9
+    qz, sz = oracle.block_weight_quant(np.zeros((128, 128), np.float32))
+    assert sz[0, 0] == 0 and not qz.any()
+
+
+# ---- the block-scaled GEMM -----------------------------------------------------------------------------
+def _rand_problem(M, N, K, seed):
+    x = H.activations(M, K, seed=seed)
+    q, s = oracle.group_quant_fp8(tr.bits_of(x))
+    wq, ws = oracle.block_weight_quant(H.weights(N, K, seed=seed + 1).float().numpy())
+    return q, s, wq, ws
+
+
+def test_gemm_brute_force_float64():
+    M, N, K = 5, 130, 256
+    q, s, wq, ws = _rand_problem(M, N, K, 40)
+    # dequantise in fp32 (as the reference's check does), multiply-accumulate in float64
+    a = (oracle.e4m3fn_to_f32(q) * np.repeat(s, 128, 1)).astype(np.float64)
+    b = (oracle.e4m3fn_to_f32(wq) * np.repeat(np.repeat(ws, 128, 0)[:N], 128, 1)).astype(np.float64)
+    want = a @ b.T
+    got64 = oracle.dequant_matmul_sampled(q, s, wq, ws, np.arange(M), np.arange(N))
+    assert np.allclose(got64, want, rtol=1e-12, atol=0)
+    bits, c32 = oracle.block_gemm(q, s, wq, ws, want_f32=True)
+    assert np.abs(c32 - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.array_equal(bits, oracle.f32_to_bf16(c32))
+    # sampling picks the right rows/columns
+    sub = oracle.dequant_matmul_sampled(q, s, wq, ws, [4, 1], [129, 0, 64])
+    assert np.array_equal(sub, got64[[4, 1]][:, [129, 0, 64]])
+
+
+def test_gemm_unit_scales_reduce_to_integer_matmul():
+    g = np.random.default_rng(41)
+    M, N, K = 7, 140, 384
+    a = g.integers(-8, 9, (M, K)).astype(np.float32)
+    b = g.integers(-8, 9, (N, K)).astype(np.float32)
+    _, c32 = oracle.block_gemm(oracle.f32_to_e4m3fn(a), np.ones((M, 3), np.float32), oracle.f32_to_e4m3fn(b),
+                               np.ones((2, 3), np.float32), want_f32=True)
+    assert np.array_equal(c32, a @ b.T)  # integers: exact in fp32
+
+
+def test_gemm_scales_enter_per_block_and_per_operand():
+    """A transposed or mis-indexed scale must fail here: distinct power-of-two scales per (row, k-block) and
+    per (n-block, k-block), integer payloads, so the expected result is exact."""
+    g = np.random.default_rng(42)
+    M, N, K = 4, 256, 256
+    a = g.integers(-4, 5, (M, K)).astype(np.float32)
+    b = g.integers(-4, 5, (N, K)).astype(np.float32)
+    As = 2.0 ** g.integers(-3, 4, (M, 2)).astype(np.float32)
+    Bs = 2.0 ** g.integers(-3, 4, (2, 2)).astype(np.float32)
+    want = np.zeros((M, N))
+    for kb in range(2):
+        blk = a[:, kb * 128:(kb + 1) * 128] @ b[:, kb * 128:(kb + 1) * 128].T
+        want += blk * As[:, kb:kb + 1] * np.repeat(Bs[:, kb], 128)[None, :]
+    _, c32 = oracle.block_gemm(oracle.f32_to_e4m3fn(a), As, oracle.f32_to_e4m3fn(b), Bs, want_f32=True)
+    assert np.array_equal(c32, want.astype(np.float32))
+
+
+def test_gemm_matches_torch_dequant_matmul_cpu_reference_config():
+    """The reference's CPU-runnable case: M=32, N=K=4096, seed 0 (fp32 dequant + matmul, bf16 out)."""
+    x = H.activations(32, 4096, seed=0)
+    xq, xs = tr.group_quant(x)
+    wq, ws = tr.block_weight_quant(H.weights(4096, 4096, seed=0))
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    bits = oracle.block_gemm(tr.bits_of(xq), xs.numpy(), tr.bits_of(wq), ws.numpy())
+    got = tr.bf16_from_bits(bits).float()
+    cos, rel = H.gemm_metrics(got, ref)
+    assert cos >= 0.99999 and rel <= 2 ** -8, (cos, rel)   # two fp32 summation orders + one bf16 rounding
+
+
+# ---- routing tables and the grouped GEMM -----------------------------------------------------------------
+def test_moe_align_fused_reference_golden():
+    """Vectors of unit_tests/common/fused_moe/test_grouped_fused_moe.py:80-126 (bincount / nonzero form)."""
+    ids = np.array([[0, 1, 2], [0, 3, 1], [3, 1, 4]], np.int32)
+    w = np.array([[0.3, 0.7, 0.1], [0.2, 0.8, 0.4], [0.5, 0.6, 0.9]], np.float32)
+    idx, ew, cnt = oracle.moe_align_fused(ids, w, 5)
+    assert cnt.tolist() == [2, 3, 1, 2, 1]
+    assert idx[0, :2].tolist() == [0, 3] and idx[1, :3].tolist() == [1, 5, 7] and idx[3, :2].tolist() == [4, 6]
+    assert np.allclose(ew[1, :3], [0.7, 0.4, 0.6])
+    ids = (np.arange(128 * 17, dtype=np.int32).reshape(128, 17) % 5)
+    idx, ew, cnt = oracle.moe_align_fused(ids, np.arange(ids.size, dtype=np.float32), 5)
+    flat = ids.ravel()
+    assert np.array_equal(cnt, np.bincount(flat, minlength=5))
+    for e in range(5):
+        want = np.nonzero(flat == e)[0]
+        assert np.array_equal(idx[e, :cnt[e]], want) and np.array_equal(ew[e, :cnt[e]], want.astype(np.float32))
+
+
+def test_moe_align1_demo_of_the_reference():
+    """The worked example in the reference's moe_align1 docstring (grouped_fused_moe.py:160-190)."""
+    idx, ew, cnt = oracle.moe_align_fused(np.array([[0, 1], [1, 3]], np.int32),
+                                          np.array([[0.3, 0.7], [0.2, 0.8]], np.float32), 4)
+    assert cnt.tolist() == [1, 2, 0, 1]
+    assert idx[0, 0] == 0 and idx[1, :2].tolist() == [1, 2] and idx[3, 0] == 3
+    assert np.allclose(ew[1, :2], [0.7, 0.2]) and np.isclose(ew[3, 0], 0.8)
+
+
+def test_moe_align2_reference_golden():
+    """unit_tests/common/fused_moe/test_grouped_fused_moe.py:219-258."""
+    t = oracle.moe_align2(100, [8, 0, 60, 16], 16)
+    assert t.shape[0] == 10
+    assert t[:, 0].tolist() == [0, 2, 2, 2, 2, 3, -1, -1, -1, -1]
+    assert t[:6, 1].tolist() == [0, 0, 1, 2, 3, 0]
+    assert t[:6, 2].tolist() == [0, 8, 24, 40, 56, 68]
+    t = oracle.moe_align2(8, [8] + [0] * 9, 16)
+    assert t.shape[0] == 8 and t[0, 0] == 0 and np.all(t[1:, 0] == -1)
+
+
+def test_grouped_gemm_is_a_per_expert_loop_of_the_dense_oracle():
+    T, E, topk, N, K = 24, 5, 3, 140, 256
+    ids, tw = H.routing(T, E, topk, seed=50)
+    idx, ew, cnt = oracle.moe_align_fused(ids.numpy(), tw.numpy(), E)
+    xq, xs = oracle.group_quant_fp8(tr.bits_of(H.activations(T, K, seed=51)))
+    Wq = np.empty((E, N, K), np.uint8)
+    Ws = np.empty((E, 2, 2), np.float32)
+    for e in range(E):
+        Wq[e], Ws[e] = oracle.block_weight_quant(H.weights(N, K, seed=60 + e).float().numpy())
+    for mul in (False, True):
+        out = oracle.grouped_block_gemm(xq, xs, Wq, Ws, idx, ew, cnt, topk, mul)
+        flat = ids.numpy().ravel()
+        for pair in range(T * topk):
+            e, row = flat[pair], pair // topk
+            _, c32 = oracle.block_gemm(xq[row:row + 1], xs[row:row + 1], Wq[e], Ws[e], want_f32=True)
+            if mul:
+                c32 = c32 * tw.numpy().ravel()[pair]
+            assert np.array_equal(out[pair], oracle.f32_to_bf16(c32[0]))
+
+
+# ---- the steps between the two expert GEMMs ---------------------------------------------------------------
+def test_silu_and_mul_and_sum_reduce_closed_forms():
+    x = H.activations(9, 512, seed=70)
+    g, u = x[:, :256].float(), x[:, 256:]
+    want = (g / (1 + torch.exp(-g))).to(torch.bfloat16) * u
+    got = tr.bf16_from_bits(oracle.silu_and_mul(tr.bits_of(x)))
+    assert (got.float() - want.float()).abs().max() <= want.float().abs().max() * 2 ** -7
+    y = H.activations(6 * 4, 128, seed=71).reshape(6, 4, 128)
+    want = y.float().sum(1).to(torch.bfloat16)
+    got = tr.bf16_from_bits(oracle.moe_sum_reduce(tr.bits_of(y.reshape(24, 128)).reshape(6, 4, 128)))
+    assert (got.float() - want.float()).abs().max() <= want.float().abs().max() * 2 ** -7
