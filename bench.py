@@ -118,7 +118,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true")
-    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|grouped (for profiling)")
+    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|prefill|grouped|copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path; this build has no multi-GPU leg (--gpus must be 1)",
@@ -291,12 +291,20 @@ def main():
             del w, wscale, xq, xs, out
             torch.cuda.empty_cache()
 
+    if args.only == "copy":
+        # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        us = _time_calls(lambda: dst.copy_(src), 5, 2)
+        others.append({"name": "copy 1 GiB (reads 2^30 B, writes 2^30 B per launch)", "us": round(us, 1),
+                       "GB/s": round(2 * (1 << 30) / us / 1e3, 1)})
+
     if not result:
         result = {"metric": "partial run (--only)", "n_gpus": 1}
     if others:
         result["others"] = others
     if run_all and not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(64, N, K)
+        result["cpu_baseline"] = cpu_baseline(512, N, K)
     print(json.dumps(result))
 
 

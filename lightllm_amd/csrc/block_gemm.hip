@@ -69,7 +69,7 @@ static int launch_dense(GemmArgs &a, hipStream_t st) {
 // Weight-streaming launch for M <= 64: tiles BM x 64, deep DMA ring, K split so that about one CTA per CU
 // streams a long run of weight bytes.
 constexpr int kSkinnyBN = 64;
-constexpr int kSkinnyStages = 8;
+constexpr int kSkinnyStages = 4;
 
 static int skinny_bm(int64_t M) { return M <= 16 ? 16 : (M <= 32 ? 32 : 64); }
 

@@ -295,33 +295,45 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     }
 
     // ---- split-K: publish the partial, let the last CTA of the tile reduce
+    // Partials and the arrival counter are exchanged with agent-scope relaxed atomics: such stores write
+    // through, and such loads read past, the per-XCD L2, so no cache-wide write-back / invalidate fence is
+    // needed (one of those per CTA costs more than the whole GEMM at decode sizes).  Order is kept by
+    // "all my stores acknowledged (vmcnt 0) -> barrier -> one atomic add" on the writer side and
+    // "atomic add returned -> barrier -> loads" on the reader side.
     if constexpr (MODE == kSplitK) {
         constexpr int kTileElems = BM * BN;
         float *mine = p.partials + ((int64_t)tile_id * p.splits + split) * kTileElems;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) *(v4f *)(mine + ((i * TN + j) * Cfg::kThreads + tid) * 4) = acc[i][j];
-        __threadfence();
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    __hip_atomic_store(mine + ((i * TN + j) * Cfg::kThreads + tid) * 4 + v, acc[i][j][v], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        wait_vmcnt<0>();
         __syncthreads();
-        // (kept in the dynamic allocation: a static __shared__ object would push static + opt-in dynamic
-        // LDS past the 160 KiB a workgroup may ask for)
+        // (the arrival word lives in the dynamic allocation: a static __shared__ object would push static +
+        // opt-in dynamic LDS past the 160 KiB a workgroup may ask for)
         volatile uint32_t *arrived = (volatile uint32_t *)(lds + Cfg::kWsOff + Cfg::NBC * KB * 4);
-        if (tid == 0) *arrived = atomicAdd(p.counters + tile_id, 1u);
+        if (tid == 0)
+            *arrived = __hip_atomic_fetch_add(p.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*arrived != (uint32_t)p.splits - 1u) return;
-        __threadfence();
         const float *base = p.partials + (int64_t)tile_id * p.splits * kTileElems;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 v4f s = v4f{0.f, 0.f, 0.f, 0.f};
-                for (int sp = 0; sp < p.splits; ++sp)
-                    s += __builtin_nontemporal_load((const v4f *)(base + (int64_t)sp * kTileElems + ((i * TN + j) * Cfg::kThreads + tid) * 4));
+                for (int sp = 0; sp < p.splits; ++sp) {
+                    const float *q = base + (int64_t)sp * kTileElems + ((i * TN + j) * Cfg::kThreads + tid) * 4;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) s[v] += __hip_atomic_load(q + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
                 acc[i][j] = s;
             }
-        if (tid == 0) p.counters[tile_id] = 0u;
+        if (tid == 0) __hip_atomic_store(p.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue: lane (r16, g4) holds, for each tm, row m = wave_m*WMS + 16*tm + r16 and the 4*TN
