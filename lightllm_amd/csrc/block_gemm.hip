@@ -1,6 +1,8 @@
 // Host side of the block-scaled FP8 GEMM entry points: argument checks, kernel choice, launches.
+#include <cstdlib>
 #include <mutex>
 
+#include "gemm_stream.hpp"
 #include "gemm_tile.hpp"
 
 namespace mi355 {
@@ -66,37 +68,60 @@ static int launch_dense(GemmArgs &a, hipStream_t st) {
     return launch_tile<BM, BN, WM, WN, NSTAGE, kDense>(a, a.blocks_per_xcd * 8, st);
 }
 
-// Weight-streaming launch for M <= 64: tiles BM x 64, deep DMA ring, K split so that about one CTA per CU
-// streams a long run of weight bytes.
-constexpr int kSkinnyBN = 64;
-constexpr int kSkinnyStages = 4;
+// Weight-streaming launch for M <= 64: 64-row tiles (16-, 32- and 128-row tiles all measured slower on the
+// decode shapes), the K range split over CTAs only as far as needed to give every CU a CTA, and never below
+// 16 K steps per CTA (4 per wave).
+static int skinny_mt(int64_t M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 
-static int skinny_bm(int64_t M) { return M <= 16 ? 16 : (M <= 32 ? 32 : 64); }
+struct SkinnyPlan {
+    int tnw, splits, tiles;
+};
 
-static int skinny_splits(int64_t N, int64_t K, int cus) {
-    const int tiles_n = (int)((N + kSkinnyBN - 1) / kSkinnyBN);
+static SkinnyPlan skinny_plan(int64_t M, int64_t N, int64_t K, int cus) {
+    (void)M;
+    SkinnyPlan pl;
+    pl.tnw = 4;
+    pl.tiles = (int)((N + 16 * pl.tnw - 1) / (16 * pl.tnw));
     const int KB = (int)(K / kBlockK);
-    int splits = (cus + tiles_n - 1) / tiles_n;        // reach at least one CTA per CU
-    const int max_splits = KB / 8 > 0 ? KB / 8 : 1;     // keep at least 8 K steps per CTA
-    if (splits > max_splits) splits = max_splits;
-    if (splits < 1) splits = 1;
-    return splits;
+    pl.splits = (cus + pl.tiles - 1) / pl.tiles;
+    const int max_splits = KB / 16 > 0 ? KB / 16 : 1;
+    if (pl.splits > max_splits) pl.splits = max_splits;
+    if (pl.splits < 1) pl.splits = 1;
+    return pl;
 }
 
-template <int BM>
-static int launch_skinny(GemmArgs &a, int splits, void *ws, hipStream_t st) {
-    constexpr int BN = kSkinnyBN;
-    a.tiles_m = 1;
-    a.tiles_n = (a.N + BN - 1) / BN;
-    a.total_tiles = a.tiles_n;
-    if (splits <= 1) {
-        a.blocks_per_xcd = (a.total_tiles + 7) / 8;
-        return launch_tile<BM, BN, 1, 4, kSkinnyStages, kDense>(a, a.blocks_per_xcd * 8, st);
+static size_t skinny_workspace(int64_t M, const SkinnyPlan &pl) {
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)pl.tiles * pl.splits * 16 * skinny_mt(M) * 16 * pl.tnw * 4;
+}
+
+template <int MT, int TNW>
+static int launch_stream(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStream_t st) {
+    using Cfg = StreamCfg<MT, TNW>;
+    static std::once_flag once;
+    static hipError_t e0 = hipSuccess, e1 = hipSuccess;
+    std::call_once(once, [&] {
+        e0 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, false>, Cfg::kLds);
+        e1 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, true>, Cfg::kLds);
+    });
+    if (e0 != hipSuccess || e1 != hipSuccess) return MI355_ELAUNCH;
+    if (pl.splits <= 1) {
+        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, false>), dim3(pl.tiles), dim3(256), Cfg::kLds, st, a);
+    } else {
+        a.splits = pl.splits;
+        a.counters = (uint32_t *)ws;
+        a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, true>), dim3(pl.tiles * pl.splits), dim3(256), Cfg::kLds,
+                           st, a);
     }
-    a.splits = splits;
-    a.counters = (uint32_t *)ws;
-    a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
-    return launch_tile<BM, BN, 1, 4, kSkinnyStages, kSplitK>(a, a.total_tiles * splits, st);
+    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+}
+
+template <int MT>
+static int launch_stream_mt(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStream_t st) {
+    switch (pl.tnw) {
+        case 4: return launch_stream<MT, 4>(a, pl, ws, st);
+        default: return MI355_EINVAL;
+    }
 }
 
 static int device_cus() {
@@ -119,8 +144,24 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 static int pick_variant(int64_t M, int64_t N, int cus) {
     if (M <= 64) return MI355_GEMM_SKINNY;
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (t256 >= (int64_t)cus * 3 / 4) return MI355_GEMM_TILE256;
+    if (t256 >= (int64_t)cus / 2) return MI355_GEMM_TILE256;
     return MI355_GEMM_TILE128;
+}
+
+// 128x128 tiles that are too few to occupy the device share the K range: about one CTA per CU, at least
+// 8 K steps each.
+static int tile128_splits(int64_t M, int64_t N, int64_t K, int cus) {
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    const int64_t KB = K / kBlockK;
+    if (tiles * 2 > cus || KB < 16) return 1;
+    int64_t splits = cus / tiles;
+    if (splits > KB / 8) splits = KB / 8;
+    return (int)(splits < 1 ? 1 : splits);
+}
+
+static size_t tile128_workspace(int64_t M, int64_t N, int splits) {
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 128 * 128 * 4;
 }
 
 }  // namespace mi355
@@ -130,13 +171,14 @@ using namespace mi355;
 extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, 256);
-    if (variant != MI355_GEMM_SKINNY || M > 64 || K % kBlockK != 0) return 0;
-    // sized for the largest split any device would pick, so the figure does not depend on the device
-    const int64_t tiles = (N + kSkinnyBN - 1) / kSkinnyBN;
-    int64_t max_splits = K / kBlockK / 8;
-    if (max_splits < 1) max_splits = 1;
-    if (tiles * 4 > MI355_WS_COUNTER_BYTES) return 0;
-    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * max_splits * skinny_bm(M) * kSkinnyBN * 4;
+    if (K % kBlockK != 0) return 0;
+    if (variant == MI355_GEMM_TILE128) {
+        const int splits = tile128_splits(M, N, K, 256);
+        return splits > 1 ? tile128_workspace(M, N, splits) * 2 : 0;  // x2: headroom for devices with more CUs
+    }
+    if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
+    // sized for the deepest split (a one-CU device), so the figure does not depend on the device
+    return skinny_workspace(M, skinny_plan(M, N, K, 1 << 20));
 }
 
 extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C,
@@ -193,21 +235,30 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
             return launch_dense<256, 256, 2, 4, 2>(a, st);
         case MI355_GEMM_TILE256x128:
             return launch_dense<256, 128, 2, 4, 3>(a, st);
-        case MI355_GEMM_TILE128:
-            return launch_dense<128, 128, 2, 2, 2>(a, st);
+        case MI355_GEMM_TILE128: {
+            const int splits = tile128_splits(M, N, K, cus);
+            if (splits <= 1 || !ws || ws_bytes < tile128_workspace(M, N, splits) || ((uintptr_t)ws & 15))
+                return launch_dense<128, 128, 2, 2, 2>(a, st);  // without a workspace the split is simply not used
+            a.tiles_m = (a.M + 127) / 128;
+            a.tiles_n = (a.N + 127) / 128;
+            a.total_tiles = a.tiles_m * a.tiles_n;
+            a.splits = splits;
+            a.counters = (uint32_t *)ws;
+            a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+            return launch_tile<128, 128, 2, 2, 2, kSplitK>(a, a.total_tiles * splits, st);
+        }
         case MI355_GEMM_SKINNY: {
             if (M > 64) return MI355_EUNSUPPORTED;
-            const int splits = skinny_splits(N, K, cus);
-            if (splits > 1) {
-                const size_t need = (size_t)MI355_WS_COUNTER_BYTES +
-                                    (size_t)((N + kSkinnyBN - 1) / kSkinnyBN) * splits * skinny_bm(M) * kSkinnyBN * 4;
-                if (!ws || ws_bytes < need || ((uintptr_t)ws & 15)) return MI355_EWORKSPACE;
-                if (((N + kSkinnyBN - 1) / kSkinnyBN) * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
-            }
-            switch (skinny_bm(M)) {
-                case 16: return launch_skinny<16>(a, splits, ws, st);
-                case 32: return launch_skinny<32>(a, splits, ws, st);
-                default: return launch_skinny<64>(a, splits, ws, st);
+            // the stream kernel addresses rows from the matrix bases with 32-bit byte offsets
+            if (N * ldb_n >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)) return MI355_EUNSUPPORTED;
+            const SkinnyPlan pl = skinny_plan(M, N, K, cus);
+            if ((int64_t)pl.tiles * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
+            if (pl.splits > 1 && (!ws || ws_bytes < skinny_workspace(M, pl) || ((uintptr_t)ws & 15)))
+                return MI355_EWORKSPACE;
+            switch (skinny_mt(M)) {
+                case 1: return launch_stream_mt<1>(a, pl, ws, st);
+                case 2: return launch_stream_mt<2>(a, pl, ws, st);
+                default: return launch_stream_mt<4>(a, pl, ws, st);
             }
         }
         default:

@@ -93,9 +93,12 @@ def grouped_matmul(
     assert expert_weights.is_contiguous()
     assert expert_to_weights_scale is not None and expert_to_weights_scale.ndim == 3
     assert expert_to_weights_scale.is_contiguous() and out.is_contiguous()
-    block_size_n = expert_weights.shape[1] // expert_to_weights_scale.shape[1]
-    block_size_k = expert_weights.shape[2] // expert_to_weights_scale.shape[2]
-    assert block_size_n == 128 and block_size_k == 128, "weights must be 128x128 block-quantized"
+    # 128x128 weight blocks (the reference derives the block sizes from the two shapes, :814-816; the last
+    # n block may be partial here)
+    block_size_k = 128
+    assert expert_to_weights_scale.shape[1] == (n + 127) // 128 and expert_to_weights_scale.shape[2] * 128 == k, (
+        "weights must be 128x128 block-quantized"
+    )
     assert out.dtype == torch.bfloat16 and out.shape[1] == n
     _lib.require_cuda(token_inputs, expert_weights, out)
     lib = _lib.lib()

@@ -112,6 +112,23 @@ def test_one_hot_rows_pick_scaled_columns(hip):
         assert torch.all((got - ref).abs() <= ref.abs() * 2 ** -7 + 1e-30), variant
 
 
+@pytest.mark.parametrize("M,N,K", [(128, 512, 4096), (200, 640, 8192), (65, 256, 2048)])
+def test_mid_m_split_k_tiles(hip, M, N, K):
+    """Few 128x128 tiles and a long K: the tiled kernel shares the K range between CTAs."""
+    print(f"gemm mid-M split-K M={M} N={N} K={K}", flush=True)
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + K)
+    C1 = _run(xq, xs, wq, ws, None).clone()
+    C2 = _run(xq, xs, wq, ws, "tile128").clone()
+    assert torch.equal(C1, C2) and torch.equal(C2, _run(xq, xs, wq, ws, "tile128"))
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(C1.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+    rows, cols = np.arange(0, M, 7), np.arange(0, N, 5)
+    ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq), xs.cpu().numpy(), tr.bits_of(wq), ws.cpu().numpy(), rows, cols)
+    got = C1[rows][:, cols].float().cpu().double().numpy()
+    assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
+
+
 def test_split_k_is_deterministic_and_reusable(hip):
     """The split-K path reduces in a fixed order and leaves its workspace counters zero: repeated calls agree bit for bit."""
     print("gemm split-k determinism", flush=True)
