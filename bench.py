@@ -197,7 +197,11 @@ def main():
                 "peak": FP8_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
-                "traffic": None,
+                # HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0), factors from
+                # a 1 GiB device copy: 1629.2 MB read + 302.6 MB written
+                # (profiles/gemm_tile256_deepseek_gate_up_M4096.md)
+                "traffic": 1.9318e9,
+                "algorithmic_bytes_per_launch": gemm_bytes(M, N, K),
                 "launch_us": round(gemm_us, 2),
                 "algorithmic_flops_per_launch": flops,
                 "peak_derived_from_device": round(derived_peak, 1),
