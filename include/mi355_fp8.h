@@ -149,6 +149,47 @@ int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W,
                                  int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
                                  void *stream);
 
+/* ---- element-wise steps between / after the two expert GEMMs ------------------------------------------------ */
+
+/*
+ * out[m, h] = bf16( bf16(silu(in[m, h])) * in[m, H + h] ),  silu(g) = g / (1 + exp(-g)) in fp32.
+ * in bf16 [M, 2H] = [gate | up] with row stride in_stride_m (elements), out bf16 [M, H] with row stride out_stride_m.
+ * Replaces: silu_and_mul_fwd(input, output, layout="blocked")
+ *           (lightllm/common/basemodel/triton_kernel/fused_moe/moe_silu_and_mul.py:9-93, 117-176).
+ */
+int mi355_silu_and_mul(const void *in, void *out, int64_t M, int64_t H, int64_t in_stride_m, int64_t out_stride_m,
+                       void *stream);
+
+/*
+ * The same product, quantized on the fly: q e4m3fn [M, H] contiguous and one fp32 scale per 1x128 group at
+ * s[m * s_stride_m + g * s_stride_g]; arithmetic of mi355_group_quant_fp8 with eps = 1e-10 applied to the bf16
+ * products, so the result equals mi355_silu_and_mul followed by mi355_group_quant_fp8 byte for byte.
+ * masked_m == NULL: every row.  masked_m != NULL: the M rows are M / rows_per_expert experts of rows_per_expert
+ * rows each and only the first masked_m[e] rows of expert e are computed; other rows of q and s are not written.
+ * Replaces: silu_and_mul_masked_post_quant_fwd(input, output, output_scale, quant_group_size, masked_m)
+ *           (lightllm/common/basemodel/triton_kernel/fused_moe/moe_silu_and_mul_mix_quant_ep.py:9-141), and the
+ *           pair silu_and_mul_fwd + per_token_group_quant_fp8 inside fused_experts_impl
+ *           (fused_moe/grouped_fused_moe.py:1084-1090 and :862-875).
+ */
+int mi355_silu_and_mul_group_quant_fp8(const void *in, void *q, float *s, int64_t M, int64_t H, int64_t in_stride_m,
+                                       int32_t group, int64_t s_stride_m, int64_t s_stride_g,
+                                       const int32_t *masked_m, int64_t rows_per_expert, void *stream);
+
+/*
+ * out[t, h] = bf16( sum_k in[t, k, h] ), fp32 accumulation in ascending k.  in bf16 [T, topk, H], out bf16 [T, H],
+ * both contiguous.
+ * Replaces: moe_sum_reduce(input, output) (lightllm/common/basemodel/triton_kernel/fused_moe/moe_sum_reduce.py:8-108).
+ */
+int mi355_moe_sum_reduce(const void *in, void *out, int64_t T, int32_t topk, int64_t H, void *stream);
+
+/*
+ * out[n, k] = bf16( float(q[n, k]) * s[n / 128, k / 128] ).  q e4m3fn [N, K] contiguous, s fp32
+ * [ceil(N/128), ceil(K/128)] contiguous, out bf16 [N, K] contiguous.  The inverse of the block weight quantizer.
+ * Replaces: weight_dequant(x, s, block_size=128) (lightllm/models/deepseek2/triton_kernel/weight_dequant.py:9-59).
+ */
+int mi355_block_weight_dequant(const void *q, const float *s, void *out, int64_t N, int64_t K, int32_t block,
+                               void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -34,6 +34,12 @@ SIGNATURES = {
         _c.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp],
     ),
+    "mi355_silu_and_mul": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "mi355_silu_and_mul_group_quant_fp8": (
+        _c.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i64, _i64, _vp, _i64, _vp]
+    ),
+    "mi355_moe_sum_reduce": (_c.c_int, [_vp, _vp, _i64, _i32, _i64, _vp]),
+    "mi355_block_weight_dequant": (_c.c_int, [_vp, _vp, _vp, _i64, _i64, _i32, _vp]),
 }
 
 _lib = None

@@ -20,17 +20,16 @@ constexpr int kBlockN = 128;
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
 
-// fp32 -> bf16 bits, round to nearest even (finite inputs).
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t u = as_u32(f);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
-}
+// fp32 -> bf16 bits, round to nearest even, NaN kept a NaN: gfx950 converts two floats per instruction
+// (v_cvt_pk_bf16_f32).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    uint32_t a = as_u32(lo), b = as_u32(hi);
-    a += 0x7fffu + ((a >> 16) & 1u);
-    b += 0x7fffu + ((b >> 16) & 1u);
-    return (a >> 16) | (b & 0xffff0000u);
+    v2f v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    return (uint32_t)__builtin_bit_cast(unsigned short, (__bf16)f);
 }
 
 // D(16x16, fp32) = A(16x128, e4m3) * B(128x16, e4m3) + C on the CDNA4 matrix core.

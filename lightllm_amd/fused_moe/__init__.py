@@ -1,1 +1,7 @@
-from .grouped_fused_moe import grouped_matmul, moe_align2, moe_align_fused  # noqa: F401
+from .grouped_fused_moe import fused_experts_impl, grouped_matmul, moe_align2, moe_align_fused  # noqa: F401
+from .moe_silu_and_mul import silu_and_mul_fwd  # noqa: F401
+from .moe_silu_and_mul_mix_quant_ep import (  # noqa: F401
+    silu_and_mul_masked_post_quant_fwd,
+    silu_and_mul_post_quant_fwd,
+)
+from .moe_sum_reduce import moe_sum_reduce  # noqa: F401

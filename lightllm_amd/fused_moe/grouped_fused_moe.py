@@ -2,8 +2,8 @@
 
 Same names, arguments and tensor layouts as
 lightllm/common/basemodel/triton_kernel/fused_moe/grouped_fused_moe.py of the reference
-(moe_align_fused :388-396, moe_align2 :452-477, grouped_matmul :771-989); the work is done by
-``mi355_moe_align_fused``, ``mi355_moe_align2`` and ``mi355_grouped_block_fp8_gemm``.
+(moe_align_fused :388-396, moe_align2 :452-477, grouped_matmul :771-989, fused_experts_impl :992-1115);
+the work is done by ``mi355_moe_align_fused``, ``mi355_moe_align2`` and ``mi355_grouped_block_fp8_gemm``.
 Only the fp8 128x128-block branch exists here (use_fp8_w8a8=True with 3-D weight scales).
 """
 from typing import Optional
@@ -12,8 +12,11 @@ import torch
 
 from .. import _lib
 from ..quantization.fp8act_quant_kernel import per_token_group_quant_fp8
+from .moe_silu_and_mul_mix_quant_ep import silu_and_mul_post_quant_fwd
+from .moe_sum_reduce import moe_sum_reduce
 
 _BLOCK_MS = (16, 32, 64, 128)
+FFN_MOE_CHUNK_SIZE = 32 * 1024  # tokens per pass of fused_experts_impl (reference :34)
 
 
 def moe_align_fused(expert_to_token_index, expert_to_weight, expert_token_num, topk_ids, topk_weights):
@@ -130,3 +133,89 @@ def grouped_matmul(
     )
     _lib.check(code, "grouped_matmul")
     return (table, block_m)
+
+
+def fused_experts_impl(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    inplace: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    w1_bias: Optional[torch.Tensor] = None,
+    w2_bias: Optional[torch.Tensor] = None,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    alloc_tensor_func=torch.empty,
+    run_config: Optional[dict] = None,
+    layout="blocked",
+    limit=None,
+    alpha=None,
+):
+    """The routed-expert FFN: out[t] = sum_k w[t,k] * ( silu_mul( x[t] @ w1[e].T ) @ w2[e].T ),  e = topk_ids[t,k].
+
+    hidden_states bf16 [T, H]; w1 e4m3fn [E, 2I, H] (gate rows then up rows), w2 e4m3fn [E, H, I];
+    w1_scale / w2_scale fp32 128x128-block scales; topk_ids int32 [T, topk], topk_weights fp32 [T, topk].
+
+    Same steps and the same results as the reference's sequence (routing tables, gate/up GEMM,
+    silu_and_mul, quantize, down GEMM with the routed weight, sum over slots); the SiLU product is
+    quantized where it is produced, so its bf16 form [T*topk, I] is never written to memory.
+    """
+    assert use_fp8_w8a8 and not use_int8_w8a16, "only the fp8 block-quantized branch is implemented on gfx950"
+    assert w1_bias is None and w2_bias is None, "per-expert bias is not supported by the fp8 block branch"
+    if layout != "blocked" or limit is not None or alpha is not None:
+        raise ValueError("fused_experts_impl: only layout='blocked' without limit/alpha is implemented on gfx950")
+    assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype == torch.bfloat16
+    num_tokens, _ = hidden_states.shape
+    E, N, _ = w1.shape
+    assert N % 256 == 0 and w2.shape[2] == N // 2, "intermediate size must be a multiple of 128"
+    topk_num = topk_ids.shape[1]
+    M = min(num_tokens, FFN_MOE_CHUNK_SIZE)
+    device, dtype = hidden_states.device, hidden_states.dtype
+
+    # gate/up output and down output share one buffer, as in the reference: the first is dead once quantized
+    shared13 = alloc_tensor_func((M, topk_num, max(N, w2.shape[1])), device=device, dtype=dtype)
+    cache1 = shared13.view(-1)[: M * topk_num * N].view(M, topk_num, N)
+    cache3 = shared13.view(-1)[: M * topk_num * w2.shape[1]].view(M, topk_num, w2.shape[1])
+    cache2_q = alloc_tensor_func((M, topk_num, N // 2), device=device, dtype=torch.float8_e4m3fn)
+    cache2_s = alloc_tensor_func((M, topk_num, N // 2 // 128), device=device, dtype=torch.float32)
+
+    out_hidden_states = hidden_states if inplace else alloc_tensor_func(hidden_states.shape, device=device, dtype=dtype)
+
+    for begin in range(0, num_tokens, FFN_MOE_CHUNK_SIZE):
+        end = min(begin + FFN_MOE_CHUNK_SIZE, num_tokens)
+        cur = hidden_states[begin:end]
+        tokens = end - begin
+        c1, c3 = cache1[:tokens], cache3[:tokens]
+        c2_q, c2_s = cache2_q[:tokens], cache2_s[:tokens]
+        cur_ids, cur_weights = topk_ids[begin:end], topk_weights[begin:end]
+        pairs = cur_ids.numel()
+
+        expert_to_tokens = torch.empty((E, pairs), dtype=torch.int32, device=device)
+        expert_to_weights = torch.empty((E, pairs), dtype=torch.float32, device=device)
+        expert_to_token_num = torch.empty((E,), dtype=torch.int32, device=device)
+        moe_align_fused(expert_to_tokens, expert_to_weights, expert_to_token_num, cur_ids, cur_weights)
+
+        reused = grouped_matmul(
+            pairs, cur, a1_scale, expert_to_token_num, expert_to_tokens, expert_to_weights=expert_to_weights,
+            expert_weights=w1, expert_to_weights_scale=w1_scale, topk_num=topk_num, out=c1.view(-1, N),
+            mul_routed_weight=False, use_fp8_w8a8=True, alloc_tensor_func=alloc_tensor_func, run_config=run_config,
+        )
+        silu_and_mul_post_quant_fwd(c1.view(-1, N), c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128))
+        grouped_matmul(
+            pairs, c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128), expert_to_token_num, expert_to_tokens,
+            expert_to_weights=expert_to_weights, expert_weights=w2, expert_to_weights_scale=w2_scale, topk_num=1,
+            out=c3.view(-1, w2.shape[1]), mul_routed_weight=True, use_fp8_w8a8=True,
+            alloc_tensor_func=alloc_tensor_func, reused_mblock_infos=reused, run_config=run_config,
+        )
+        moe_sum_reduce(c3, out_hidden_states[begin:end])
+    return out_hidden_states

@@ -199,3 +199,34 @@ def moe_sum_reduce(x_bf16_bits) -> np.ndarray:
     out = np.empty((T, H), np.uint16)
     lib().oracle_moe_sum_reduce(_p(x), I64(T), I32(topk), I64(H), _p(out))
     return out
+
+
+def block_weight_dequant(q_bytes, scales, block: int = 128) -> np.ndarray:
+    q, sc = _c(q_bytes, np.uint8), _c(scales, np.float32)
+    N, K = q.shape
+    assert sc.shape == ((N + block - 1) // block, (K + block - 1) // block)
+    out = np.empty((N, K), np.uint16)
+    lib().oracle_block_weight_dequant(_p(q), _p(sc), I64(N), I64(K), I32(block), _p(out))
+    return out
+
+
+def silu_and_mul_group_quant(x_bf16_bits, group: int = 128):
+    """silu_and_mul followed by the group quantizer: what the fused kernel must reproduce
+    (fused_moe/moe_silu_and_mul_mix_quant_ep.py:51-74 repeats the quantizer's arithmetic on the bf16 product)."""
+    return group_quant_fp8(silu_and_mul(x_bf16_bits), group)
+
+
+def fused_experts(x_bf16_bits, w1_q, w1_s, w2_q, w2_s, topk_ids, topk_weights) -> np.ndarray:
+    """The routed-expert FFN as the reference sequences it (fused_moe/grouped_fused_moe.py:1048-1113):
+    routing tables, quantize, gate/up grouped GEMM, silu_and_mul, quantize, down grouped GEMM times the routed
+    weight, sum over slots.  x bf16 bits [T,H]; w1 e4m3 bytes [E,2I,H]; w2 [E,H,I] -> bf16 bits [T,H]."""
+    x = _c(x_bf16_bits, np.uint16)
+    ids = _c(topk_ids, np.int32)
+    T, topk = ids.shape
+    E = w1_q.shape[0]
+    idx, ew, cnt = moe_align_fused(ids, topk_weights, E)
+    xq, xs = group_quant_fp8(x)
+    h1 = grouped_block_gemm(xq, xs, w1_q, w1_s, idx, ew, cnt, topk, False)
+    aq, as_ = silu_and_mul_group_quant(h1)
+    h3 = grouped_block_gemm(aq, as_, w2_q, w2_s, idx, ew, cnt, 1, True)
+    return moe_sum_reduce(h3.reshape(T, topk, -1))

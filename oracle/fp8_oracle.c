@@ -19,7 +19,9 @@
  *   oracle_block_gemm*          pinned: unit-scale / one-hot special cases, numpy f64
  *   oracle_moe_align_fused/2    pinned: the reference's own golden vectors
  *   oracle_grouped_block_gemm   pinned: per-expert loop of the dense oracle
- *   oracle_silu_and_mul*        pinned: torch closed form
+ *   oracle_silu_and_mul         pinned: torch closed form (bit-equal but for rare 1-ulp exp differences), special values
+ *   oracle_moe_sum_reduce       pinned: exactly summable inputs, torch closed form
+ *   oracle_block_weight_dequant pinned: torch closed form, round trip through oracle_block_weight_quant
  */
 #include <math.h>
 #include <stdint.h>
@@ -355,9 +357,19 @@ void oracle_moe_sum_reduce(const uint16_t *in, int64_t T, int32_t topk, int64_t 
         }
 }
 
+/* weight_dequant (models/deepseek2/triton_kernel/weight_dequant.py:9-59): out[n,k] = bf16( f32(q[n,k]) * s[n/block, k/block] ). */
+void oracle_block_weight_dequant(const uint8_t *q, const float *s, int64_t N, int64_t K, int32_t block, uint16_t *out) {
+    const int64_t kb = (K + block - 1) / block;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t k = 0; k < K; ++k) {
+            volatile float y = oracle_e4m3fn_to_f32(q[n * K + k]) * s[(n / block) * kb + k / block];
+            out[n * K + k] = oracle_f32_to_bf16(y);
+        }
+}
+
 /*
  * Replays, on the CPU, the exact operation sequence the HIP quantizer uses in place of two IEEE
- * divisions (csrc/group_quant.hip: quant_chunk/quot), for every bf16 group maximum with bit pattern in
+ * divisions (csrc/quant_core.hpp: quant_chunk/quot), for every bf16 group maximum with bit pattern in
  * [amax_lo, amax_hi) stepping by `step`, against every bf16 element of either sign with |x| <= amax
  * (and every |x| < eps when the eps floor applies).  Returns how many (amax, x) pairs give a byte or a
  * scale different from the IEEE closed form above.  Zero for the whole range means the kernel's

@@ -272,14 +272,87 @@ def test_grouped_gemm_is_a_per_expert_loop_of_the_dense_oracle():
             assert np.array_equal(out[pair], oracle.f32_to_bf16(c32[0]))
 
 
-# ---- the steps between the two expert GEMMs ---------------------------------------------------------------
-def test_silu_and_mul_and_sum_reduce_closed_forms():
-    x = H.activations(9, 512, seed=70)
-    g, u = x[:, :256].float(), x[:, 256:]
-    want = (g / (1 + torch.exp(-g))).to(torch.bfloat16) * u
-    got = tr.bf16_from_bits(oracle.silu_and_mul(tr.bits_of(x)))
-    assert (got.float() - want.float()).abs().max() <= want.float().abs().max() * 2 ** -7
+# ---- the steps between and after the two expert GEMMs --------------------------------------------------------
+def test_silu_and_mul_special_values():
+    """silu(0) = 0, silu(g) = g for large g (1 + exp(-g) rounds to 1), silu(g) = -0 for g << 0, silu(1) known."""
+    H2 = 8
+    gate = torch.tensor([0.0, 20.0, 64.0, -100.0, 1.0, -1.0, 3.0, 88.0]).to(torch.bfloat16)
+    up = torch.tensor([3.0, 0.5, -2.0, 7.0, 1.0, 1.0, 1.0, 1.0]).to(torch.bfloat16)
+    x = torch.cat([gate, up]).reshape(1, 2 * H2)
+    got = tr.bf16_from_bits(oracle.silu_and_mul(tr.bits_of(x))).float().reshape(-1)
+    assert got[0] == 0.0 and got[1] == 10.0 and got[2] == -128.0 and got[3] == 0.0
+    # silu(1) = 0.7310585..., silu(-1) = -0.2689414..., silu(3) = 2.8577223...: rounded to bf16
+    for i, v in ((4, 0.7310585786300049), (5, -0.2689414213699951), (6, 2.857722300624436)):
+        assert got[i] == torch.tensor(v).to(torch.bfloat16).float()
+    assert got[7] == 88.0
+
+
+def test_silu_and_mul_matches_torch_float64_rounding():
+    """Against silu evaluated in float64 and rounded once to fp32 then bf16: the oracle's fp32 evaluation may
+    differ by an fp32 ulp before the bf16 rounding, which flips at most a handful of bf16 results by one ulp."""
+    x = H.activations(64, 1024, seed=70)
+    x = (x.float() * 3).to(torch.bfloat16)
+    g, u = x[:, :512].double(), x[:, 512:]
+    a = (g / (1 + torch.exp(-g))).float().to(torch.bfloat16)
+    want = tr.bits_of((a.float() * u.float()).to(torch.bfloat16)).astype(np.int32)
+    got = oracle.silu_and_mul(tr.bits_of(x)).astype(np.int32)
+    diff = np.abs(got - want)
+    assert diff.max() <= 1 or np.all((got[diff > 1] & 0x7fff) < 0x80)   # beyond one ulp only between tiny values
+    assert (diff != 0).mean() < 1e-3
+
+
+def test_moe_sum_reduce_exact_and_ordered():
+    # integers: every partial sum is exact, any order gives the same answer
+    g = H.gen(71)
+    y = torch.randint(-64, 64, (6, 8, 128), generator=g).to(torch.bfloat16)
+    got = tr.bf16_from_bits(oracle.moe_sum_reduce(tr.bits_of(y)))
+    assert torch.equal(got, y.float().sum(1).to(torch.bfloat16))
+    # order matters in fp32: 2^24 + 1 - 2^24 summed left to right is 0, not 1
+    z = torch.zeros((1, 3, 8), dtype=torch.float32)
+    z[0, 0], z[0, 1], z[0, 2] = 2.0 ** 24, 1.0, -(2.0 ** 24)
+    got = tr.bf16_from_bits(oracle.moe_sum_reduce(tr.bits_of(z.to(torch.bfloat16))))
+    assert torch.all(got.float() == 0.0)
+    # torch closed form
     y = H.activations(6 * 4, 128, seed=71).reshape(6, 4, 128)
-    want = y.float().sum(1).to(torch.bfloat16)
-    got = tr.bf16_from_bits(oracle.moe_sum_reduce(tr.bits_of(y.reshape(24, 128)).reshape(6, 4, 128)))
-    assert (got.float() - want.float()).abs().max() <= want.float().abs().max() * 2 ** -7
+    want = y[:, 0].float()
+    for k in range(1, 4):
+        want = want + y[:, k].float()
+    got = tr.bf16_from_bits(oracle.moe_sum_reduce(tr.bits_of(y)))
+    assert torch.equal(got, want.to(torch.bfloat16))
+
+
+def test_block_weight_dequant_closed_form_and_round_trip():
+    w = H.weights(200, 300, seed=72)
+    q, s = tr.block_weight_quant(w)
+    want = (q.float() * s.repeat_interleave(128, 0)[:200].repeat_interleave(128, 1)[:, :300]).to(torch.bfloat16)
+    got = tr.bf16_from_bits(oracle.block_weight_dequant(tr.bits_of(q), s.numpy()))
+    assert torch.equal(got, want)
+    # inverse of the quantizer up to the e4m3 step (2^-4 relative, half of it after rounding) plus the bf16 step
+    rel = (got.float() - w.float()).abs() / w.float().abs().clamp_min(1e-3)
+    assert rel.max() < 0.07
+
+
+def test_fused_experts_composition_against_dense_float():
+    """The oracle's routed-expert FFN against the plain per-token loop over dequantized weights in fp32
+    (the structure of fused_experts_impl_ref, unit_tests/common/fused_moe/test_deepep.py:59-140)."""
+    T, Hd, I, E, topk = 12, 256, 128, 6, 2
+    x = H.activations(T, Hd, seed=73)
+    w1 = H.weights(E * 2 * I, Hd, seed=74).reshape(E, 2 * I, Hd)
+    w2 = H.weights(E * Hd, I, seed=75).reshape(E, Hd, I)
+    q1 = [tr.block_weight_quant(w1[e]) for e in range(E)]
+    q2 = [tr.block_weight_quant(w2[e]) for e in range(E)]
+    ids, tw = H.routing(T, E, topk, seed=76)
+    out = oracle.fused_experts(
+        tr.bits_of(x), np.stack([tr.bits_of(q) for q, _ in q1]), np.stack([s.numpy() for _, s in q1]),
+        np.stack([tr.bits_of(q) for q, _ in q2]), np.stack([s.numpy() for _, s in q2]), ids.numpy(), tw.numpy())
+    got = tr.bf16_from_bits(out).float()
+    want = torch.zeros((T, Hd))
+    for t in range(T):
+        for k in range(topk):
+            e = int(ids[t, k])
+            d1, d2 = tr.dequant(*q1[e], 128, 128), tr.dequant(*q2[e], 128, 128)
+            h = x[t].float() @ d1.T
+            a = torch.nn.functional.silu(h[:I]) * h[I:]
+            want[t] += tw[t, k] * (a @ d2.T)
+    assert tr.cosine(got, want) > 0.999
+    assert (got - want).abs().max() / want.abs().max() < 0.05
