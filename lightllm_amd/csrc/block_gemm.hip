@@ -49,7 +49,8 @@ static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
     auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE>;
     const int KB = a.K / kBlockK;
-    const int lds_bytes = Cfg::lds_bytes(KB);
+    // the ping-pong kernel keeps two [BM rows][8 steps] chunks of X scales behind the common layout
+    const int lds_bytes = MODE == kDensePP ? ((Cfg::lds_bytes(KB) + 127) & ~127) + 2 * BM * 32 : Cfg::lds_bytes(KB);
     if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -59,13 +60,13 @@ static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE = kDense>
 static int launch_dense(GemmArgs &a, hipStream_t st) {
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (a.N + BN - 1) / BN;
     a.total_tiles = a.tiles_m * a.tiles_n;
     a.blocks_per_xcd = (a.total_tiles + 7) / 8;
-    return launch_tile<BM, BN, WM, WN, NSTAGE, kDense>(a, a.blocks_per_xcd * 8, st);
+    return launch_tile<BM, BN, WM, WN, NSTAGE, MODE>(a, a.blocks_per_xcd * 8, st);
 }
 
 // Weight-streaming launch for M <= 64: 64-row tiles (16-, 32- and 128-row tiles all measured slower on the
@@ -231,7 +232,13 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
     a.vec_store = (((uintptr_t)C & 15) == 0 && ldc % 8 == 0 && N % 8 == 0) ? 1 : 0;
 
     switch (variant) {
-        case MI355_GEMM_TILE256:
+        case MI355_GEMM_TILE256: {
+            // the ping-pong kernel fetches X scales eight K steps at a time: row-major scales, 16-byte aligned rows
+            const bool chunked_scales = as_k == 1 && (K / kBlockK) % 8 == 0 && as_m % 4 == 0 && ((uintptr_t)As & 15) == 0;
+            if (chunked_scales) return launch_dense<256, 256, 2, 4, 2, kDensePP>(a, st);
+            return launch_dense<256, 256, 2, 4, 2>(a, st);
+        }
+        case 6:  // the plain ring kernel on the 256x256 tile, whatever the scale layout (kept for comparison)
             return launch_dense<256, 256, 2, 4, 2>(a, st);
         case MI355_GEMM_TILE256x128:
             return launch_dense<256, 128, 2, 4, 3>(a, st);

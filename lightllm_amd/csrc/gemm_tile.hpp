@@ -36,7 +36,7 @@
 
 namespace mi355 {
 
-enum { kDense = 0, kGrouped = 1, kSplitK = 2 };
+enum { kDense = 0, kGrouped = 1, kSplitK = 2, kDensePP = 3 };
 
 struct GemmArgs {
     const uint8_t *X;    // [M,K] (dense) or [T,K] (grouped), row stride ldx bytes
@@ -250,48 +250,173 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     }
     const int nk = kb_end - kb_begin;
 
-    // prologue: fill NSTAGE-1 stages
+    if constexpr (MODE == kDensePP) {
+        // Two-group ping-pong with early refill, for the 256x256 tile (8 waves, two ring slots).
+        //
+        // The 8 waves form two groups (waves 0-3 and 4-7: one wave of each group per SIMD) that run the same
+        // phase sequence one phase apart, so while one group's waves keep the matrix pipe busy the other
+        // group's waves fetch operands from LDS and feed the DMA.  Phases of one K step, a barrier after each:
+        //   A0  read the W fragments and the first half of the X fragments (+ their scales)
+        //   B0  MFMA + scale fold of the first half
+        //   A1  read the second half of the X fragments (+ scales)
+        //   B1  MFMA + scale fold of the second half
+        // Group 1 starts one barrier late and group 0 ends one barrier late, so both count the same number.
+        //
+        // The pipeline is bound by the L2 -> LDS path, so a region of a ring slot is refilled as soon as both
+        // groups have read it instead of once per step: the W rows and the first-half X rows of tile it+2 are
+        // requested at the top of A1(it) (into the slot tile it is leaving), the second-half X rows of tile
+        // it+1 at the top of A0(it).  Every request is waited for one and a half steps later, by every wave,
+        // before the barrier that lets the first group read it.  The loop body has no branches (steps past the
+        // end re-fetch the last tile, identical bytes) so that the phases stay where they are written.
+        //
+        // X scales.  Fetching one column of the row-major [M, K/128] scale matrix per step costs one cache
+        // line per row and step - as many L2 requests as the tile itself.  Instead a [256 rows][8 steps] chunk
+        // is fetched at a time (32 useful bytes per line) into one of two LDS buffers: 16 lanes per wave and
+        // step, during the first four steps of the previous chunk (the last four steps repeat those requests;
+        // identical bytes).  Needs K/128 % 8 == 0, unit k stride and 16-byte aligned scale rows.
+        static_assert(NSTAGE == 2 && Cfg::kWaves == 8 && TM % 2 == 0 && Cfg::XI == 4 && BM == 256, "ping-pong layout");
+        constexpr int HM = TM / 2;
+        constexpr int kXhi = Cfg::XI / 2 + 1;          // requests per wave at the top of A0 (X second half + scale piece)
+        constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;   // requests per wave at the top of A1
+        const int grp = wave >> 2;
+        const uint32_t chunk0 = lds0 + (uint32_t)((Cfg::lds_bytes(KB) + 127) & ~127);
+        auto phase_end = [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8)); };
+        // piece j (0..3) of the scale chunk starting at step kc: rows 64*j + 8*wave + lane/2, 4 steps per lane
+        auto issue_scales = [&](int buf, int j, int kc) {
+            const int row = j * 64 + wave * 8 + ((lane & 15) >> 1);
+            const uint32_t voff = (uint32_t)(min(row, rows_valid - 1) * (int)p.xs_m + 4 * (lane & 1)) * 4u;
+            if (lane < 16)
+                dma_g2l_b128(chunk0 + (uint32_t)buf * (BM * 32) + (uint32_t)(j * 128 + wave * 16) * 16u, sg + kc, voff);
+        };
+        auto issue_wxlo = [&](int stage, int kb) {
+            const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
+            const uint8_t *xk = xg + (int64_t)kb * kBlockK;
+            const uint8_t *wk = wg + (int64_t)kb * kBlockK;
 #pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s)
-        if (s < nk) issue(s, kb_begin + s);
-
-    int cur = 0;            // ring slot of step it
-    int fill = NSTAGE - 1;  // ring slot the next DMA goes to
-    for (int it = 0; it < nk; ++it) {
-        // stage `it` must have landed; the NSTAGE-2 stages issued after it may still be in flight
-        if (it + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * Cfg::kLoadsPerStage>();
-        else wait_vmcnt<0>();
+            for (int i = 0; i < Cfg::XI; i += 2) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+#pragma unroll
+            for (int i = 0; i < Cfg::WI; ++i) dma_g2l_b128(sb + wdst[i], wk, woff[i]);
+        };
+        auto issue_xhi = [&](int stage, int kb) {
+            const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
+            const uint8_t *xk = xg + (int64_t)kb * kBlockK;
+#pragma unroll
+            for (int i = 1; i < Cfg::XI; i += 2) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+        };
+        const int nchunk = KB / 8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) issue_scales(0, j, 0);
+        issue_wxlo(0, 0);
+        issue_xhi(0, 0);
+        issue_wxlo(1, min(1, nk - 1));
+        wait_vmcnt<kWXlo>();
         __syncthreads();
-        if (it + NSTAGE - 1 < nk) issue(fill, kb_begin + it + NSTAGE - 1);
-        const float ws_cur = wsl[kb_begin + it];
-
-        const uint8_t *st = lds + cur * Cfg::kStage;
-        float xs[TM];
-        {
-            const float *sp = (const float *)(lds + sr + cur * (BM * 4));
-#pragma unroll
-            for (int i = 0; i < TM; ++i) xs[i] = sp[i] * ws_cur;
-        }
-        v8i wf[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
-            const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
-            wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
-            const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
-            const v8i xf = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        if (grp == 1) phase_end();
+        // scale of (row, step) sits at chunk[(step/8) & 1][row][step % 8]
+        const uint32_t sr8 = (uint32_t)((Cfg::lds_bytes(KB) + 127) & ~127) + (uint32_t)(wave_m * WMS + r16) * 32u;
+        int cur = 0;
+        for (int it = 0; it < nk; ++it) {
+            const uint8_t *st = lds + cur * Cfg::kStage;
+            const int cbuf = (it >> 3) & 1;
+            // ---- A0
+            issue_xhi(cur ^ 1, min(it + 1, nk - 1));
+            issue_scales(cbuf ^ 1, it & 3, 8 * min((it >> 3) + 1, nchunk - 1));
+            const float ws_cur = wsl[it];
+            const float *sp = (const float *)(lds + sr8 + cbuf * (BM * 32) + (it & 7) * 4);
+            v8i wf[TN], xf[HM];
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const v4f part = mfma_16x16x128_fp8(wf[j], xf, v4f{0.f, 0.f, 0.f, 0.f});
-                acc[i][j] += part * xs[i];
+                const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
+                const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
+                wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (h == 1) issue_wxlo(cur, min(it + 2, nk - 1));
+                float xs[HM];
+#pragma unroll
+                for (int i = 0; i < HM; ++i) {
+                    const v4i lo = *(const v4i *)(st + xr0 + (h * HM + i) * 2048);
+                    const v4i hi = *(const v4i *)(st + xr1 + (h * HM + i) * 2048);
+                    xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    xs[i] = sp[(h * HM + i) * 16 * 8] * ws_cur;
+                }
+                // everything but the last two request groups has landed: at the end of A0 that covers the second
+                // X half of this tile, at the end of A1 the W rows and first X half of the next one
+                wait_vmcnt<kXhi + kWXlo>();
+                wait_lds();
+                phase_end();
+                // ---- B0 / B1: the scale fold of one product runs behind the next product's MFMA
+                __builtin_amdgcn_s_setprio(1);
+                v4f prev = mfma_16x16x128_fp8(wf[0], xf[0], v4f{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                for (int e = 1; e < HM * TN; ++e) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    const v4f part = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
+                    acc[h * HM + (e - 1) / TN][(e - 1) % TN] += prev * xs[(e - 1) / TN];
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
+                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // the previous product's fold behind it
+                    prev = part;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                acc[h * HM + HM - 1][TN - 1] += prev * xs[HM - 1];
+                __builtin_amdgcn_s_setprio(0);
+                phase_end();
+            }
+            cur ^= 1;
         }
-        cur = cur + 1 == NSTAGE ? 0 : cur + 1;
-        fill = fill + 1 == NSTAGE ? 0 : fill + 1;
+        if (grp == 0) phase_end();
+        wait_vmcnt<0>();  // the re-fetches of the last steps must not outlive the workgroup's LDS
+    } else {
+        // prologue: fill NSTAGE-1 stages
+#pragma unroll
+        for (int s = 0; s < NSTAGE - 1; ++s)
+            if (s < nk) issue(s, kb_begin + s);
+
+        int cur = 0;            // ring slot of step it
+        int fill = NSTAGE - 1;  // ring slot the next DMA goes to
+        for (int it = 0; it < nk; ++it) {
+            // stage `it` must have landed; the NSTAGE-2 stages issued after it may still be in flight
+            if (it + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * Cfg::kLoadsPerStage>();
+            else wait_vmcnt<0>();
+            __syncthreads();
+            if (it + NSTAGE - 1 < nk) issue(fill, kb_begin + it + NSTAGE - 1);
+            const float ws_cur = wsl[kb_begin + it];
+
+            const uint8_t *st = lds + cur * Cfg::kStage;
+            float xs[TM];
+            {
+                const float *sp = (const float *)(lds + sr + cur * (BM * 4));
+    #pragma unroll
+                for (int i = 0; i < TM; ++i) xs[i] = sp[i] * ws_cur;
+            }
+            v8i wf[TN];
+    #pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
+                const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
+                wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+    #pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
+                const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
+                const v8i xf = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    #pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const v4f part = mfma_16x16x128_fp8(wf[j], xf, v4f{0.f, 0.f, 0.f, 0.f});
+                    acc[i][j] += part * xs[i];
+                }
+            }
+            cur = cur + 1 == NSTAGE ? 0 : cur + 1;
+            fill = fill + 1 == NSTAGE ? 0 : fill + 1;
+        }
+
     }
 
     // ---- split-K: publish the partial, let the last CTA of the tile reduce
