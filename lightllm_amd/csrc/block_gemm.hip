@@ -44,13 +44,18 @@ static hipError_t allow_lds(KernelT kernel, int bytes) {
     return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
-static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
+// X scales that can be fetched eight K steps at a time: row-major, 16-byte aligned rows, K/128 % 8 == 0.
+static bool chunked_scales_ok(const GemmArgs &a) {
+    return a.xs_k == 1 && (a.K / kBlockK) % 8 == 0 && a.xs_m % 4 == 0 && ((uintptr_t)a.Xs & 15) == 0;
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
+static int launch_tile_as(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
-    auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE>;
+    auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE, XS8>;
     const int KB = a.K / kBlockK;
-    // the ping-pong kernel keeps two [BM rows][8 steps] chunks of X scales behind the common layout
-    const int lds_bytes = MODE == kDensePP ? ((Cfg::lds_bytes(KB) + 127) & ~127) + 2 * BM * 32 : Cfg::lds_bytes(KB);
+    // chunked scales keep two [BM rows][8 steps] buffers behind the common layout
+    const int lds_bytes = XS8 ? ((Cfg::lds_bytes(KB) + 127) & ~127) + 2 * BM * 32 : Cfg::lds_bytes(KB);
     if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -58,6 +63,23 @@ static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     if (attr_err != hipSuccess) return MI355_ELAUNCH;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::kThreads), lds_bytes, st, a);
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
+static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
+    using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
+    constexpr bool kFits = ((Cfg::lds_bytes(144) + 127) & ~127) + 2 * BM * 32 <= kMaxLds;  // up to K = 18432
+    if constexpr (MODE == kDensePP) {
+        return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
+    } else {
+        if constexpr (kFits) {
+            if (chunked_scales_ok(a)) {
+                const int r = launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
+                if (r != MI355_EUNSUPPORTED) return r;
+            }
+        }
+        return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false>(a, grid, st);
+    }
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE = kDense>
@@ -234,8 +256,7 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
     switch (variant) {
         case MI355_GEMM_TILE256: {
             // the ping-pong kernel fetches X scales eight K steps at a time: row-major scales, 16-byte aligned rows
-            const bool chunked_scales = as_k == 1 && (K / kBlockK) % 8 == 0 && as_m % 4 == 0 && ((uintptr_t)As & 15) == 0;
-            if (chunked_scales) return launch_dense<256, 256, 2, 4, 2, kDensePP>(a, st);
+            if (chunked_scales_ok(a)) return launch_dense<256, 256, 2, 4, 2, kDensePP>(a, st);
             return launch_dense<256, 256, 2, 4, 2>(a, st);
         }
         case 6:  // the plain ring kernel on the 256x256 tile, whatever the scale layout (kept for comparison)

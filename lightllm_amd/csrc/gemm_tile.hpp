@@ -75,7 +75,7 @@ struct TileCfg {
     static constexpr int XI = XG >= kWaves ? XG / kWaves : 1;  // DMA instructions per wave per stage
     static constexpr int WI = WG >= kWaves ? WG / kWaves : 1;
     static constexpr int SG = BM >= 64 ? BM / 64 : 1;          // 64-row groups of the scale vector
-    static constexpr int kLoadsPerStage = XI + WI + 1;        // identical for every wave
+    static constexpr int kLoadsPerStage = XI + WI + 1;        // identical for every wave (one less with chunked scales)
     static constexpr int kStage = (BM + BN) * 128;
     static constexpr int kScaleOff = NSTAGE * kStage;
     static constexpr int kWsOff = kScaleOff + NSTAGE * BM * 4;  // weight scales of the whole K range
@@ -89,9 +89,13 @@ struct TileCfg {
     static_assert(NSTAGE >= 2 && (NSTAGE - 2) * kLoadsPerStage < 64, "vmcnt is a 6-bit counter");
 };
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
+// XS8: the X scales are row-major with 16-byte aligned rows and K/128 % 8 == 0, so they are fetched as
+// [BM rows][8 steps] chunks (one request per 64 half-rows and chunk) instead of one column per step.
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
 __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const GemmArgs p) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
+    static_assert(MODE != kDensePP || XS8, "the ping-pong schedule needs chunked scales");
+    constexpr int kLoads = Cfg::XI + Cfg::WI + (XS8 ? 0 : 1);  // DMA requests per wave and stage
     constexpr int TM = Cfg::TM, TN = Cfg::TN, WMS = Cfg::WMS, WNS = Cfg::WNS;
     constexpr bool GROUPED = MODE == kGrouped;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -222,9 +226,36 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         for (int i = 0; i < Cfg::WI; ++i) dma_g2l_b128(sb + wdst[i], wk, woff[i]);
         // every wave issues this (waves beyond the tile repeat a group) so that all waves count the same
         // number of outstanding loads per stage; lanes past the tile's rows stay idle
-        if (s_active)
-            dma_g2l_b32(lds0 + Cfg::kScaleOff + (uint32_t)stage * (BM * 4) + sdst, sg + (int64_t)kb * p.xs_k, soff);
+        if constexpr (!XS8) {
+            if (s_active)
+                dma_g2l_b32(lds0 + Cfg::kScaleOff + (uint32_t)stage * (BM * 4) + sdst, sg + (int64_t)kb * p.xs_k, soff);
+        }
     };
+
+    // Chunked X scales (XS8).  Fetching one column of the row-major [M, K/128] scale matrix per step costs one
+    // cache line per row and step - as many L2 requests as the X tile itself.  Instead a [BM rows][8 steps]
+    // chunk is fetched at a time (32 useful bytes per line) into one of two LDS buffers behind the common
+    // layout: lane l of wave w fetches steps 4*(l&1).. of row 32*w + l/2.  The scale of (row, step kb) then sits
+    // at chunk[(kb/8) & 1][row][kb % 8].
+    constexpr uint32_t kChunkBytes = BM * 32;
+    const uint32_t chunk_off = (uint32_t)((Cfg::lds_bytes(KB) + 127) & ~127);
+    uint32_t sc_off = 0;
+    const bool sc_active = XS8 && wave * 64 + lane < 2 * BM;
+    if (sc_active) {
+        const int rc = min(wave * 32 + (lane >> 1), rows_valid - 1);
+        uint32_t src_row;
+        if constexpr (GROUPED) src_row = (uint32_t)idx_list[m0 + rc] / (uint32_t)p.topk;
+        else src_row = (uint32_t)rc;
+        sc_off = (src_row * (uint32_t)p.xs_m + 4u * (uint32_t)(lane & 1)) * 4u;
+    }
+    auto issue_scales = [&](int chunk) {
+        if (wave * 64 < 2 * BM) {
+            if (sc_active)
+                dma_g2l_b128(lds0 + chunk_off + (uint32_t)(chunk & 1) * kChunkBytes + (uint32_t)wave * 1024u, sg + 8 * chunk, sc_off);
+        }
+    };
+    const int nchunk = KB / 8;
+    const uint32_t sr8 = chunk_off + (uint32_t)(wave_m * WMS + r16) * 32u;
 
     // ---- per-lane LDS read offsets
     const uint32_t fr = swz((uint32_t)r16);
@@ -269,30 +300,19 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         // before the barrier that lets the first group read it.  The loop body has no branches (steps past the
         // end re-fetch the last tile, identical bytes) so that the phases stay where they are written.
         //
-        // X scales.  Fetching one column of the row-major [M, K/128] scale matrix per step costs one cache
-        // line per row and step - as many L2 requests as the tile itself.  Instead a [256 rows][8 steps] chunk
-        // is fetched at a time (32 useful bytes per line) into one of two LDS buffers: 16 lanes per wave and
-        // step, during the first four steps of the previous chunk (the last four steps repeat those requests;
-        // identical bytes).  Needs K/128 % 8 == 0, unit k stride and 16-byte aligned scale rows.
+        // The X scales come in [256 rows][8 steps] chunks (see issue_scales), requested in the first step of
+        // the previous chunk.
         static_assert(NSTAGE == 2 && Cfg::kWaves == 8 && TM % 2 == 0 && Cfg::XI == 4 && BM == 256, "ping-pong layout");
         constexpr int HM = TM / 2;
-        constexpr int kXhi = Cfg::XI / 2 + 1;          // requests per wave at the top of A0 (X second half + scale piece)
-        constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;   // requests per wave at the top of A1
+        constexpr int kXhi = Cfg::XI / 2;              // requests per wave in A0 (X second half)
+        constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;   // requests per wave in A1
         const int grp = wave >> 2;
-        const uint32_t chunk0 = lds0 + (uint32_t)((Cfg::lds_bytes(KB) + 127) & ~127);
         auto phase_end = [&]() {
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
         };
         auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8)); };
-        // piece j (0..3) of the scale chunk starting at step kc: rows 64*j + 8*wave + lane/2, 4 steps per lane
-        auto issue_scales = [&](int buf, int j, int kc) {
-            const int row = j * 64 + wave * 8 + ((lane & 15) >> 1);
-            const uint32_t voff = (uint32_t)(min(row, rows_valid - 1) * (int)p.xs_m + 4 * (lane & 1)) * 4u;
-            if (lane < 16)
-                dma_g2l_b128(chunk0 + (uint32_t)buf * (BM * 32) + (uint32_t)(j * 128 + wave * 16) * 16u, sg + kc, voff);
-        };
         auto issue_wxlo = [&](int stage, int kb) {
             const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
             const uint8_t *xk = xg + (int64_t)kb * kBlockK;
@@ -308,26 +328,20 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
 #pragma unroll
             for (int i = 1; i < Cfg::XI; i += 2) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
         };
-        const int nchunk = KB / 8;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) issue_scales(0, j, 0);
+        issue_scales(0);
         issue_wxlo(0, 0);
         issue_xhi(0, 0);
         issue_wxlo(1, min(1, nk - 1));
         wait_vmcnt<kWXlo>();
         __syncthreads();
         if (grp == 1) phase_end();
-        // scale of (row, step) sits at chunk[(step/8) & 1][row][step % 8]
-        const uint32_t sr8 = (uint32_t)((Cfg::lds_bytes(KB) + 127) & ~127) + (uint32_t)(wave_m * WMS + r16) * 32u;
         int cur = 0;
         for (int it = 0; it < nk; ++it) {
             const uint8_t *st = lds + cur * Cfg::kStage;
             const int cbuf = (it >> 3) & 1;
-            // ---- A0
-            issue_xhi(cur ^ 1, min(it + 1, nk - 1));
-            issue_scales(cbuf ^ 1, it & 3, 8 * min((it >> 3) + 1, nchunk - 1));
+            // ---- A0 (LDS reads first: a DMA request can stall the wave's issue, the reads behind it would wait)
             const float ws_cur = wsl[it];
-            const float *sp = (const float *)(lds + sr8 + cbuf * (BM * 32) + (it & 7) * 4);
+            const float *sp = (const float *)(lds + sr8 + cbuf * kChunkBytes + (it & 7) * 4);
             v8i wf[TN], xf[HM];
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
@@ -337,7 +351,6 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             }
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                if (h == 1) issue_wxlo(cur, min(it + 2, nk - 1));
                 float xs[HM];
 #pragma unroll
                 for (int i = 0; i < HM; ++i) {
@@ -346,13 +359,19 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
                     xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     xs[i] = sp[(h * HM + i) * 16 * 8] * ws_cur;
                 }
+                if (h == 0) {
+                    if ((it & 7) == 0 && (it >> 3) + 1 < nchunk) issue_scales((it >> 3) + 1);
+                    issue_xhi(cur ^ 1, min(it + 1, nk - 1));
+                } else {
+                    issue_wxlo(cur, min(it + 2, nk - 1));
+                }
                 // everything but the last two request groups has landed: at the end of A0 that covers the second
-                // X half of this tile, at the end of A1 the W rows and first X half of the next one
+                // X half of this tile, at the end of A1 the W rows and first X half of the next one (the scale
+                // request of every eighth step only makes the wait one request stricter)
                 wait_vmcnt<kXhi + kWXlo>();
                 wait_lds();
                 phase_end();
                 // ---- B0 / B1: the scale fold of one product runs behind the next product's MFMA
-                __builtin_amdgcn_s_setprio(1);
                 v4f prev = mfma_16x16x128_fp8(wf[0], xf[0], v4f{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
                 for (int e = 1; e < HM * TN; ++e) {
@@ -365,7 +384,6 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 acc[h * HM + HM - 1][TN - 1] += prev * xs[HM - 1];
-                __builtin_amdgcn_s_setprio(0);
                 phase_end();
             }
             cur ^= 1;
@@ -373,7 +391,11 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         if (grp == 0) phase_end();
         wait_vmcnt<0>();  // the re-fetches of the last steps must not outlive the workgroup's LDS
     } else {
-        // prologue: fill NSTAGE-1 stages
+        // prologue: the scale chunk of the first step and the one after it, then NSTAGE-1 stages
+        if constexpr (XS8) {
+            issue_scales(kb_begin >> 3);
+            if ((kb_begin >> 3) + 1 < nchunk) issue_scales((kb_begin >> 3) + 1);
+        }
 #pragma unroll
         for (int s = 0; s < NSTAGE - 1; ++s)
             if (s < nk) issue(s, kb_begin + s);
@@ -382,32 +404,42 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         int fill = NSTAGE - 1;  // ring slot the next DMA goes to
         for (int it = 0; it < nk; ++it) {
             // stage `it` must have landed; the NSTAGE-2 stages issued after it may still be in flight
-            if (it + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * Cfg::kLoadsPerStage>();
+            // (a scale-chunk request in between only makes the wait stricter: requests retire in order)
+            if (it + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * kLoads>();
             else wait_vmcnt<0>();
             __syncthreads();
+            const int kb = kb_begin + it;
+            if constexpr (XS8) {
+                // the buffer of chunk kb/8 + 1 was last read in step kb - 1, before the barrier above
+                if ((kb & 7) == 0 && it > 0 && (kb >> 3) + 1 < nchunk) issue_scales((kb >> 3) + 1);
+            }
             if (it + NSTAGE - 1 < nk) issue(fill, kb_begin + it + NSTAGE - 1);
             const float ws_cur = wsl[kb_begin + it];
 
             const uint8_t *st = lds + cur * Cfg::kStage;
             float xs[TM];
-            {
+            if constexpr (XS8) {
+                const float *sp = (const float *)(lds + sr8 + ((kb >> 3) & 1) * kChunkBytes + (kb & 7) * 4);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) xs[i] = sp[i * 16 * 8] * ws_cur;
+            } else {
                 const float *sp = (const float *)(lds + sr + cur * (BM * 4));
-    #pragma unroll
+#pragma unroll
                 for (int i = 0; i < TM; ++i) xs[i] = sp[i] * ws_cur;
             }
             v8i wf[TN];
-    #pragma unroll
+#pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
                 const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
                 wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
                 const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
                 const v8i xf = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    #pragma unroll
+#pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     const v4f part = mfma_16x16x128_fp8(wf[j], xf, v4f{0.f, 0.f, 0.f, 0.f});
                     acc[i][j] += part * xs[i];
