@@ -192,7 +192,7 @@ def main():
             },
             "roofline": {
                 "bound": "mfma",
-                "kernel": "block_fp8_gemm_tile_kernel<256,256,2,4,2,dense>",
+                "kernel": "block_fp8_gemm_tile_kernel<256,256,2,4,2,ping-pong>",
                 "achieved": round(achieved, 1),
                 "peak": FP8_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
