@@ -69,7 +69,7 @@ template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
 static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
     constexpr bool kFits = ((Cfg::lds_bytes(144) + 127) & ~127) + 2 * BM * 32 <= kMaxLds;  // up to K = 18432
-    if constexpr (MODE == kDensePP) {
+    if constexpr (MODE == kDensePP || MODE == kGroupedPP) {
         return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
     } else {
         if constexpr (kFits) {
@@ -364,6 +364,9 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
         case 32: return launch_tile<32, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
         case 64: return launch_tile<64, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
         case 128: return launch_tile<128, 128, 2, 2, 2, kGrouped>(a, finish(128), st);
+        case 256:
+            if (!chunked_scales_ok(a)) return MI355_EUNSUPPORTED;
+            return launch_tile<256, 256, 2, 4, 2, kGroupedPP>(a, finish(256), st);
         default: return MI355_EINVAL;
     }
 }

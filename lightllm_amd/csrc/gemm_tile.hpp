@@ -36,7 +36,7 @@
 
 namespace mi355 {
 
-enum { kDense = 0, kGrouped = 1, kSplitK = 2, kDensePP = 3 };
+enum { kDense = 0, kGrouped = 1, kSplitK = 2, kDensePP = 3, kGroupedPP = 4 };
 
 struct GemmArgs {
     const uint8_t *X;    // [M,K] (dense) or [T,K] (grouped), row stride ldx bytes
@@ -94,10 +94,11 @@ struct TileCfg {
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
 __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const GemmArgs p) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
-    static_assert(MODE != kDensePP || XS8, "the ping-pong schedule needs chunked scales");
+    constexpr bool PINGPONG = MODE == kDensePP || MODE == kGroupedPP;
+    static_assert(!PINGPONG || XS8, "the ping-pong schedule needs chunked scales");
     constexpr int kLoads = Cfg::XI + Cfg::WI + (XS8 ? 0 : 1);  // DMA requests per wave and stage
     constexpr int TM = Cfg::TM, TN = Cfg::TN, WMS = Cfg::WMS, WNS = Cfg::WNS;
-    constexpr bool GROUPED = MODE == kGrouped;
+    constexpr bool GROUPED = MODE == kGrouped || MODE == kGroupedPP;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     // ---- which tile (and which K range)
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     }
     const int nk = kb_end - kb_begin;
 
-    if constexpr (MODE == kDensePP) {
+    if constexpr (PINGPONG) {
         // Two-group ping-pong with early refill, for the 256x256 tile (8 waves, two ring slots).
         //
         // The 8 waves form two groups (waves 0-3 and 4-7: one wave of each group per SIMD) that run the same
@@ -304,13 +305,21 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         // the previous chunk.
         static_assert(NSTAGE == 2 && Cfg::kWaves == 8 && TM % 2 == 0 && Cfg::XI == 4 && BM == 256, "ping-pong layout");
         constexpr int HM = TM / 2;
+        // Ragged (grouped) tiles: a wave whose 64-row half holds no valid row skips that half's LDS reads and
+        // MFMAs (never the barriers or the DMA requests, which every wave must count alike).  Dense tiles keep
+        // the branch-free body.
+        constexpr bool SKIP = GROUPED;
+        const bool do_half0 = !SKIP || wave_m * WMS < rows_valid;
+        const bool do_half1 = !SKIP || wave_m * WMS + WMS / 2 < rows_valid;
         constexpr int kXhi = Cfg::XI / 2;              // requests per wave in A0 (X second half)
         constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;   // requests per wave in A1
         const int grp = wave >> 2;
         auto phase_end = [&]() {
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler only: no LDS access may move across the barrier
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
+            __atomic_signal_fence(__ATOMIC_SEQ_CST);
         };
         auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8)); };
         auto issue_wxlo = [&](int stage, int kb) {
@@ -343,21 +352,26 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             const float ws_cur = wsl[it];
             const float *sp = (const float *)(lds + sr8 + cbuf * kChunkBytes + (it & 7) * 4);
             v8i wf[TN], xf[HM];
+            if (do_half0) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
-                const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
-                wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                for (int j = 0; j < TN; ++j) {
+                    const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
+                    const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
+                    wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
             }
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
+                const bool do_half = h == 0 ? do_half0 : do_half1;
                 float xs[HM];
+                if (do_half) {
 #pragma unroll
-                for (int i = 0; i < HM; ++i) {
-                    const v4i lo = *(const v4i *)(st + xr0 + (h * HM + i) * 2048);
-                    const v4i hi = *(const v4i *)(st + xr1 + (h * HM + i) * 2048);
-                    xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    xs[i] = sp[(h * HM + i) * 16 * 8] * ws_cur;
+                    for (int i = 0; i < HM; ++i) {
+                        const v4i lo = *(const v4i *)(st + xr0 + (h * HM + i) * 2048);
+                        const v4i hi = *(const v4i *)(st + xr1 + (h * HM + i) * 2048);
+                        xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        xs[i] = sp[(h * HM + i) * 16 * 8] * ws_cur;
+                    }
                 }
                 if (h == 0) {
                     if ((it & 7) == 0 && (it >> 3) + 1 < nchunk) issue_scales((it >> 3) + 1);
@@ -372,18 +386,20 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
                 wait_lds();
                 phase_end();
                 // ---- B0 / B1: the scale fold of one product runs behind the next product's MFMA
-                v4f prev = mfma_16x16x128_fp8(wf[0], xf[0], v4f{0.f, 0.f, 0.f, 0.f});
+                if (do_half) {
+                    v4f prev = mfma_16x16x128_fp8(wf[0], xf[0], v4f{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
-                for (int e = 1; e < HM * TN; ++e) {
+                    for (int e = 1; e < HM * TN; ++e) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        const v4f part = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
+                        acc[h * HM + (e - 1) / TN][(e - 1) % TN] += prev * xs[(e - 1) / TN];
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // the previous product's fold behind it
+                        prev = part;
+                    }
                     __builtin_amdgcn_sched_barrier(0);
-                    const v4f part = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
-                    acc[h * HM + (e - 1) / TN][(e - 1) % TN] += prev * xs[(e - 1) / TN];
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
-                    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // the previous product's fold behind it
-                    prev = part;
+                    acc[h * HM + HM - 1][TN - 1] += prev * xs[HM - 1];
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                acc[h * HM + HM - 1][TN - 1] += prev * xs[HM - 1];
                 phase_end();
             }
             cur ^= 1;

@@ -15,7 +15,7 @@ from ..quantization.fp8act_quant_kernel import per_token_group_quant_fp8
 from .moe_silu_and_mul_mix_quant_ep import silu_and_mul_post_quant_fwd
 from .moe_sum_reduce import moe_sum_reduce
 
-_BLOCK_MS = (16, 32, 64, 128)
+_BLOCK_MS = (16, 32, 64, 128, 256)
 FFN_MOE_CHUNK_SIZE = 32 * 1024  # tokens per pass of fused_experts_impl (reference :34)
 
 

@@ -103,19 +103,28 @@ def test_grouped_vs_oracle(hip, block_m, mul_w, topk):
     _grouped_case(T=96 if topk > 1 else 300, E=12, topk=topk, N=384, K=512, block_m=block_m, mul_w=mul_w, seed=70)
 
 
+@pytest.mark.parametrize("mul_w,topk,T,E", [(False, 4, 200, 7), (True, 1, 900, 5), (False, 2, 40, 9)])
+def test_grouped_256_row_blocks_vs_oracle(hip, mul_w, topk, T, E):
+    """The 256x256 ping-pong tile in grouped mode (needs K % 1024 == 0): experts with fewer than 64, 64-128,
+    128-256 and more than 256 rows, so that every combination of skipped half tiles occurs; N tail (640 % 256)."""
+    print(f"grouped block_m=256 mul_w={mul_w} topk={topk} T={T} E={E}", flush=True)
+    _grouped_case(T=T, E=E, topk=topk, N=640, K=2048, block_m=256, mul_w=mul_w, seed=75)
+
+
 def test_grouped_empty_and_single_token_experts(hip):
     """More experts than tokens: most experts get no rows, some one row; N tail (200 % 128 != 0)."""
     print("grouped sparse experts", flush=True)
     _grouped_case(T=5, E=40, topk=2, N=200, K=256, block_m=None, mul_w=False, seed=80)
 
 
-def test_grouped_deepseek_shape_sampled(hip):
+@pytest.mark.parametrize("block_m", [None, 256])
+def test_grouped_deepseek_shape_sampled(hip, block_m):
     """The routed-expert config at a reduced expert count (16 of 256 experts, same N/K, Zipf routing):
     every routed row is checked against the torch fp32 dequant-matmul of its expert."""
     from lightllm_amd.fused_moe import grouped_matmul
     from lightllm_amd.quantization import per_token_group_quant_fp8
 
-    print("grouped dsv3-shaped", flush=True)
+    print(f"grouped dsv3-shaped block_m={block_m}", flush=True)
     T, E, topk, N, K = 1024, 16, 8, 4096, 7168
     ids, tw = H.routing(T, E, topk, seed=90)
     idx, w, cnt = _align(ids, tw, E)
@@ -126,7 +135,8 @@ def test_grouped_deepseek_shape_sampled(hip):
         wq[e], ws[e] = H.quantized_weights(N, K, seed=100 + e, device="cuda")
     P = T * topk
     out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
-    grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=False, use_fp8_w8a8=True)
+    grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=False, use_fp8_w8a8=True,
+                   run_config={"BLOCK_SIZE_M": block_m} if block_m else None)
     torch.cuda.synchronize()
     xq, xs = per_token_group_quant_fp8(x, 128)
     dx = tr.dequant(xq, xs, 1, 128)
