@@ -138,7 +138,8 @@ int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32
  *     out[idx, :] = bf16( blockscaled(Xq[row,:] . W[e]^T) * (mul_routed_weight ? expert_to_weight[e*num_pairs+j] : 1) )
  * Xq e4m3fn [T,K] contiguous, Xs fp32 [T,K/128] contiguous (the activation quantizer's output);
  * W e4m3fn [E,N,K] contiguous; Ws fp32 [E, ceil(N/128), K/128] contiguous; out bf16 [num_pairs, N] contiguous.
- * block_m must be one the library was built for: 16, 32, 64 or 128 (mi355_grouped_block_m() suggests one).
+ * block_m must be one the library was built for: 16, 32, 64, 128, or 256 (256 needs K % 1024 == 0 and returns
+ * MI355_EUNSUPPORTED otherwise); mi355_grouped_block_m() suggests one.
  */
 int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K);
 

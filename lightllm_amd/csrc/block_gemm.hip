@@ -296,13 +296,14 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
 
 extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K) {
     (void)N;
-    (void)K;
     if (num_experts <= 0) return 64;
     const int64_t avg = num_pairs / num_experts;
     if (avg <= 16) return 16;
     if (avg <= 32) return 32;
     if (avg <= 64) return 64;
-    return 128;
+    // prefill-size batches: the 256x256 ping-pong tile (it skips the empty 64-row halves of ragged blocks);
+    // it needs the activation scales in chunks of 8 K steps
+    return (K / kBlockK) % 8 == 0 ? 256 : 128;
 }
 
 extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,

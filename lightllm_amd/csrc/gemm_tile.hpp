@@ -322,12 +322,22 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             __atomic_signal_fence(__ATOMIC_SEQ_CST);
         };
         auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8)); };
+        // Ragged tiles: an 8-row X group past the last valid row is not fetched.  Every wave must still count
+        // the same number of requests, so a one-line request (all lanes read the first 4 bytes of X into a spare
+        // LDS area) takes its place.
+        bool x_real[Cfg::XI];
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; ++i) x_real[i] = !SKIP || ((wave + i * Cfg::kWaves) % Cfg::XG) * 8 < rows_valid;
+        auto issue_x = [&](int i, uint32_t sb, const uint8_t *xk) {
+            if (x_real[i]) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+            else dma_g2l_b32(lds0 + Cfg::kScaleOff, p.X, 0u);
+        };
         auto issue_wxlo = [&](int stage, int kb) {
             const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
             const uint8_t *xk = xg + (int64_t)kb * kBlockK;
             const uint8_t *wk = wg + (int64_t)kb * kBlockK;
 #pragma unroll
-            for (int i = 0; i < Cfg::XI; i += 2) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+            for (int i = 0; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
 #pragma unroll
             for (int i = 0; i < Cfg::WI; ++i) dma_g2l_b128(sb + wdst[i], wk, woff[i]);
         };
@@ -335,7 +345,7 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
             const uint8_t *xk = xg + (int64_t)kb * kBlockK;
 #pragma unroll
-            for (int i = 1; i < Cfg::XI; i += 2) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+            for (int i = 1; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
         };
         issue_scales(0);
         issue_wxlo(0, 0);
