@@ -118,7 +118,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true")
-    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|prefill|grouped|copy (for profiling)")
+    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|prefill|grouped|moe|copy (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path; this build has no multi-GPU leg (--gpus must be 1)",
@@ -198,9 +198,9 @@ def main():
                 "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
                 # HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0), factors from
-                # a 1 GiB device copy: 1629.2 MB read + 302.6 MB written
+                # a 1 GiB device copy: 1641.2 MB read + 308.5 MB written
                 # (profiles/gemm_tile256_deepseek_gate_up_M4096.md)
-                "traffic": 1.9318e9,
+                "traffic": 1.9497e9,
                 "algorithmic_bytes_per_launch": gemm_bytes(M, N, K),
                 "launch_us": round(gemm_us, 2),
                 "algorithmic_flops_per_launch": flops,
@@ -294,6 +294,34 @@ def main():
                            "experts_hit": experts_hit})
             del w, wscale, xq, xs, out
             torch.cuda.empty_cache()
+
+    if (run_all and not args.no_others) or args.only == "moe":
+        # the element-wise steps of the routed-expert FFN at the same size (32768 rows, intermediate 2048,
+        # hidden 7168)
+        from lightllm_amd.fused_moe import moe_sum_reduce, silu_and_mul_fwd, silu_and_mul_post_quant_fwd
+
+        Pm, Im, Hm, topk_m = 32768, 2048, 7168, 8
+        h1 = make_act(Pm, 2 * Im, 50, dev)
+        act = torch.empty((Pm, Im), dtype=torch.bfloat16, device=dev)
+        aq = torch.empty((Pm, Im), dtype=torch.float8_e4m3fn, device=dev)
+        asc = torch.empty((Pm, Im // 128), dtype=torch.float32, device=dev)
+        us = _time_calls(lambda: silu_and_mul_fwd(h1, act), 30, 5)
+        byts = Pm * Im * 6
+        others.append({"name": f"silu_and_mul [{Pm},{2 * Im}]", "us": round(us, 2), "GB/s": round(byts / us / 1e3, 1),
+                       "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
+        us = _time_calls(lambda: silu_and_mul_post_quant_fwd(h1, aq, asc), 30, 5)
+        byts = Pm * Im * 5 + Pm * (Im // 128) * 4
+        others.append({"name": f"silu_and_mul + group quant fused [{Pm},{2 * Im}]", "us": round(us, 2),
+                       "GB/s": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del h1, act, aq, asc
+        h3 = make_act(Pm, Hm, 51, dev).view(Pm // topk_m, topk_m, Hm)
+        red = torch.empty((Pm // topk_m, Hm), dtype=torch.bfloat16, device=dev)
+        us = _time_calls(lambda: moe_sum_reduce(h3, red), 30, 5)
+        byts = (Pm + Pm // topk_m) * Hm * 2
+        others.append({"name": f"moe_sum_reduce [{Pm // topk_m},{topk_m},{Hm}]", "us": round(us, 2),
+                       "GB/s": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del h3, red
+        torch.cuda.empty_cache()
 
     if args.only == "copy":
         # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size
