@@ -336,7 +336,7 @@ def main():
     if others:
         result["others"] = others
     if run_all and not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(512, N, K)
+        result["cpu_baseline"] = cpu_baseline(2048, N, K)
     print(json.dumps(result))
 
 
