@@ -73,6 +73,24 @@ def test_ragged_edges(hip, M, N, K, variant):
     _check_small(xq, xs, wq, ws, _run(xq, xs, wq, ws, variant))
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 1024), (257, 520, 1024), (700, 2112, 2048), (1024, 768, 3072)])
+def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
+    """K/128 % 8 == 0 with row-major scales takes the ping-pong schedule with chunked scale fetches; the plain ring
+    on the same 256x256 tile adds the same products in the same order, so the two must agree bit for bit.
+    Column-major scales (strides (1, M)) fall back to the ring inside the same variant."""
+    print(f"gemm ping-pong vs ring M={M} N={N} K={K}", flush=True)
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + K, device="cuda")
+    c_pp = _run(xq, xs, wq, ws, "tile256")
+    c_ring = _run(xq, xs, wq, ws, "tile256ring")
+    assert torch.equal(c_pp.view(torch.int16), c_ring.view(torch.int16))
+    xs_cm = xs.t().contiguous().t()
+    assert xs_cm.stride() == (1, M) or M == 1
+    c_cm = _run(xq, xs_cm, wq, ws, "tile256")
+    assert torch.equal(c_cm.view(torch.int16), c_ring.view(torch.int16))
+    if M * N <= 300 * 600:
+        _check_small(xq, xs, wq, ws, c_pp)
+
+
 def test_unit_scales_is_plain_matmul(hip):
     """All scales 1: the result is the plain product of the fp8 values, exact in fp32 for K=128."""
     print("gemm unit scales", flush=True)

@@ -10,7 +10,7 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("N,K", [(128, 128), (256, 384), (200, 300), (2112, 1024), (1, 1)])
+@pytest.mark.parametrize("N,K", [(128, 128), (256, 384), (200, 300), (200, 304), (2112, 1024), (1, 1), (1, 8)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_bit_exact(hip, N, K, dtype):
     from lightllm_amd.quantization import mm_weight_quant
