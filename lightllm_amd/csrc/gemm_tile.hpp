@@ -395,20 +395,25 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
                 wait_vmcnt<kXhi + kWXlo>();
                 wait_lds();
                 phase_end();
-                // ---- B0 / B1: the scale fold of one product runs behind the next product's MFMA
+                // ---- B0 / B1: the scale fold of a product is issued kLag MFMAs after its own MFMA, when the
+                // result has long left the matrix pipe (a fold right behind the next MFMA would cost 7 idle
+                // issue slots every other product)
                 if (do_half) {
-                    v4f prev = mfma_16x16x128_fp8(wf[0], xf[0], v4f{0.f, 0.f, 0.f, 0.f});
+                    constexpr int E = HM * TN, kLag = 2;
+                    v4f parts[kLag + 1];
 #pragma unroll
-                    for (int e = 1; e < HM * TN; ++e) {
+                    for (int e = 0; e < E + kLag; ++e) {
                         __builtin_amdgcn_sched_barrier(0);
-                        const v4f part = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
-                        acc[h * HM + (e - 1) / TN][(e - 1) % TN] += prev * xs[(e - 1) / TN];
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
-                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // the previous product's fold behind it
-                        prev = part;
+                        if (e < E) parts[e % (kLag + 1)] = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
+                        if (e >= kLag) {
+                            const int f = e - kLag;
+                            acc[h * HM + f / TN][f % TN] += parts[f % (kLag + 1)] * xs[f / TN];
+                        }
+                        if (e < E && e >= kLag) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
+                            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // an older product's fold behind it
+                        }
                     }
-                    __builtin_amdgcn_sched_barrier(0);
-                    acc[h * HM + HM - 1][TN - 1] += prev * xs[HM - 1];
                 }
                 phase_end();
             }
