@@ -109,6 +109,15 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         split = blockIdx.x - tile_id * (uint32_t)p.splits;
         tile_m = tile_id % (uint32_t)p.tiles_m;
         tile_n = tile_id / (uint32_t)p.tiles_m;
+    } else if constexpr (MODE == kGrouped || MODE == kGroupedPP) {
+        // The schedule table is padded with empty rows at its end and tiles differ in cost, so tiles are dealt
+        // out in launch order, n fastest: the n tiles of one m block land on different XCDs, and (tiles_n being
+        // a multiple of 8 for the usual shapes) the same weight tile of consecutive m blocks on the same XCD.
+        const uint32_t bid = blockIdx.x;
+        if (bid >= (uint32_t)p.total_tiles) return;
+        tile_m = bid / (uint32_t)p.tiles_n;
+        tile_n = bid - tile_m * (uint32_t)p.tiles_n;
+        tile_id = bid;
     } else {
         // XCD-aware order.  The hardware deals workgroup ids round-robin over the 8 XCDs; give every XCD a
         // contiguous run of logical tile ids so the tiles that share an L2 share X / W panels.
