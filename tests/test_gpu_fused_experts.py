@@ -20,7 +20,8 @@ def _experts(E, I, Hd, seed):
     return st(q for q, _ in w1), st(s for _, s in w1), st(q for q, _ in w2), st(s for _, s in w2)
 
 
-@pytest.mark.parametrize("T,E,topk,Hd,I", [(1, 8, 2, 256, 128), (48, 8, 2, 512, 256), (200, 16, 4, 1024, 256), (300, 6, 1, 256, 384)])
+@pytest.mark.parametrize("T,E,topk,Hd,I", [(1, 8, 2, 256, 128), (48, 8, 2, 512, 256), (200, 16, 4, 1024, 256), (300, 6, 1, 256, 384),
+                                           (512, 4, 2, 1024, 1024)])  # the last one takes the 256-row ping-pong blocks
 def test_fused_experts_vs_oracle(hip, T, E, topk, Hd, I):
     from lightllm_amd.fused_moe import fused_experts_impl
 
