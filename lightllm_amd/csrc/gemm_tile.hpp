@@ -13,24 +13,29 @@
 //   lane then holds ONE token row m and 4 weight rows n, so the per-token scale is one register per lane
 //   and the scale fold is 4 v_fmac per MFMA:   acc += partial * (Xs[m,kb] * Ws[nb,kb]).
 //
-// LDS (dynamic): NSTAGE stages of { X tile BM x 128 B, W tile BN x 128 B }, then NSTAGE x BM floats
-//   of X scales, then the tile's weight scales for every K step (K/128 floats per 128-wide n block).  Rows are 128 B = 8 chunks of 16 B, chunk position XOR-swizzled with the row number
-//   (swz() in common.hpp) so the ds_read_b128 operand fetches are conflict free.  W rows are stored in
-//   the order the MFMA wants them: LDS row 16*tn + 4*g + v of a wave span holds weight row
-//   4*TN*g + 4*tn + v, which makes every lane's 4*TN outputs contiguous in n (one or two 16-byte stores).
-//   Tiles are filled with global_load_lds_dwordx4 (no register staging); each 8-lane group fetches one
-//   full 128-byte row segment.
+// LDS (dynamic): NSTAGE stages of { X tile BM x 128 B, W tile BN x 128 B }, then NSTAGE x BM floats of X
+//   scales (one column per stage), then the tile's weight scales for every K step (K/128 floats per 128-wide
+//   n block), then - with chunked scales - two [BM rows][8 steps] buffers of X scales.
+//   Rows are 128 B = 8 chunks of 16 B, chunk position XOR-swizzled with the row number (swz() in common.hpp)
+//   so the ds_read_b128 operand fetches are conflict free.  W rows are stored in the order the MFMA wants
+//   them: LDS row 16*tn + 4*g + v of a wave span holds weight row 4*TN*g + 4*tn + v, which makes every lane's
+//   4*TN outputs contiguous in n (one or two 16-byte stores).  Tiles are filled with global_load_lds_dwordx4
+//   (no register staging); each 8-lane group fetches one full 128-byte row segment.
 //
-// Pipeline: a ring of NSTAGE stages; the DMA for step kb+NSTAGE-1 is issued at the top of step kb, right
-//   after the one barrier of the step (which also proves that the slot being refilled has been read by all).
+// Pipelines
+//   ring       NSTAGE stages; the DMA for step kb+NSTAGE-1 is issued at the top of step kb, right after the
+//              one barrier of the step (which also proves that the slot being refilled has been read by all).
+//   ping-pong  the 256x256 tile only: two wave groups run LDS phases and MFMA phases one phase apart, ring
+//              slot regions are refilled as soon as both groups have read them (see the kernel body).
 //
 // Launch modes
-//   kDense   one CTA per output tile, whole K.
-//   kSplitK  grid = tiles x splits; each CTA accumulates a K range, stores its fp32 partial to the
-//            workspace in register order, and the CTA that arrives last at the tile's counter adds the
-//            partials in split order (deterministic), writes bf16 and re-zeroes the counter.
-//   kGrouped rows are gathered through expert_to_token_index, the tile list is the moe_align2 table, the
-//            weight and its scales are offset by the expert, rows are scattered back on store.
+//   kDense     one CTA per output tile, whole K, ring.
+//   kSplitK    grid = tiles x splits; each CTA accumulates a K range, stores its fp32 partial to the
+//              workspace in register order, and the CTA that arrives last at the tile's counter adds the
+//              partials in split order (deterministic), writes bf16 and re-zeroes the counter.
+//   kGrouped   rows are gathered through expert_to_token_index, the tile list is the moe_align2 table, the
+//              weight and its scales are offset by the expert, rows are scattered back on store.
+//   kDensePP / kGroupedPP   the dense and the grouped launch on the ping-pong pipeline.
 #pragma once
 #include "common.hpp"
 
