@@ -9,3 +9,4 @@ from .weight_dequant import weight_dequant  # noqa: F401
 from .quantize_method import QuantizationMethod, WeightPack  # noqa: F401
 from .registry import QUANTMETHODS  # noqa: F401
 from .w8a8 import FP8w8a8B128Mi355QuantizationMethod, FP8w8a8B128QuantizationMethod  # noqa: F401
+from .quantcfg import EXPERT_DTYPE_TO_QUANT_TYPE, SUPPORTED_EXPERT_DTYPES, Quantcfg  # noqa: F401
