@@ -138,6 +138,8 @@ int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32
  *     out[idx, :] = bf16( blockscaled(Xq[row,:] . W[e]^T) * (mul_routed_weight ? expert_to_weight[e*num_pairs+j] : 1) )
  * Xq e4m3fn [T,K] contiguous, Xs fp32 [T,K/128] contiguous (the activation quantizer's output);
  * W e4m3fn [E,N,K] contiguous; Ws fp32 [E, ceil(N/128), K/128] contiguous; out bf16 [num_pairs, N] contiguous.
+ * num_pairs is only used as the row stride of expert_to_token_index / expert_to_weight (the number of (token, slot)
+ * pairs in LightLLM's use); the masked expert-parallel layout passes a [E, T_pad] table with num_pairs = T_pad.
  * block_m must be one the library was built for: 16, 32, 64, 128, or 256 (256 needs K % 1024 == 0 and returns
  * MI355_EUNSUPPORTED otherwise); mi355_grouped_block_m() suggests one.
  */

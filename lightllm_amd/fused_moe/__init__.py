@@ -5,3 +5,8 @@ from .moe_silu_and_mul_mix_quant_ep import (  # noqa: F401
     silu_and_mul_post_quant_fwd,
 )
 from .moe_sum_reduce import moe_sum_reduce  # noqa: F401
+from .grouped_fused_moe_ep import (  # noqa: F401
+    _deepgemm_grouped_fp8_nt_masked,
+    deepgemm_grouped_fp8_nt_contiguous,
+    masked_group_gemm,
+)
