@@ -119,9 +119,10 @@ def test_quantization_method_surface():
     """The plug-in object exposes what LightLLM's MMWeightTpl calls (quantize_method.py:25-149, w8a8.py:418-533)."""
     from lightllm_amd.quantization import QUANTMETHODS, QuantizationMethod, WeightPack
 
-    cls = QUANTMETHODS._quant_methods["fp8w8a8-b128"]["cuda"]
+    cls = type(QUANTMETHODS.get("fp8w8a8-b128"))
     assert issubclass(cls, QuantizationMethod)
-    assert QUANTMETHODS._quant_methods["fp8w8a8-b128-triton"]["cuda"] is cls
+    assert type(QUANTMETHODS.get("fp8w8a8-b128-triton", platform="cuda")) is cls
+    assert QUANTMETHODS.get("fp8w8a8-b128") is not QUANTMETHODS.get("fp8w8a8-b128")   # a fresh object per lookup
     with pytest.raises(ValueError):
         QUANTMETHODS.get("no-such-method")
     with pytest.raises(ValueError):
