@@ -102,11 +102,12 @@ def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     callers that capture HIP graphs must run each shape once before capturing (as with any torch allocator use).
     """
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr(device))
-    buf = _workspaces.get(key)
-    if buf is None or buf.numel() < nbytes:
-        size = max(nbytes, WS_COUNTER_BYTES + (32 << 20))
-        buf = torch.zeros(size, dtype=torch.uint8, device=device)
-        _workspaces[key] = buf
+    with _lock:
+        buf = _workspaces.get(key)
+        if buf is None or buf.numel() < nbytes:
+            size = max(nbytes, WS_COUNTER_BYTES + (32 << 20))
+            buf = torch.zeros(size, dtype=torch.uint8, device=device)
+            _workspaces[key] = buf
     return buf
 
 

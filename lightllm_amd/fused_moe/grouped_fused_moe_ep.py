@@ -11,6 +11,7 @@ grouped_fused_moe_ep.py: ``_deepgemm_grouped_fp8_nt_masked`` :584-595, ``deepgem
 Weights are e4m3fn [E, N, K] with fp32 128x128-block scales [E, ceil(N/128), K/128]; outputs are bf16.
 Rows that belong to no expert (past masked_m, or m_indices < 0) are not written.
 """
+import collections
 from typing import Tuple
 
 import torch
@@ -19,7 +20,8 @@ from .. import _lib
 from .grouped_fused_moe import _BLOCK_MS, moe_align2, moe_align_fused
 from .moe_silu_and_mul_mix_quant_ep import silu_and_mul_masked_post_quant_fwd
 
-_row_tables = {}
+_row_tables = collections.OrderedDict()   # (E, T, device) -> table; the few shapes a server uses, oldest dropped
+_ROW_TABLES_KEPT = 8
 
 
 def _masked_row_table(E: int, T: int, device: torch.device) -> torch.Tensor:
@@ -29,6 +31,10 @@ def _masked_row_table(E: int, T: int, device: torch.device) -> torch.Tensor:
     if t is None:
         t = torch.arange(E * T, dtype=torch.int32, device=device).view(E, T).contiguous()
         _row_tables[key] = t
+        while len(_row_tables) > _ROW_TABLES_KEPT:
+            _row_tables.popitem(last=False)
+    else:
+        _row_tables.move_to_end(key)
     return t
 
 
