@@ -117,26 +117,39 @@ static size_t skinny_workspace(int64_t M, const SkinnyPlan &pl) {
     return (size_t)MI355_WS_COUNTER_BYTES + (size_t)pl.tiles * pl.splits * 16 * skinny_mt(M) * 16 * pl.tnw * 4;
 }
 
-template <int MT, int TNW>
-static int launch_stream(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStream_t st) {
+template <int MT, int TNW, bool XSL>
+static int launch_stream_as(GemmArgs &a, const SkinnyPlan &pl, void *ws, int lds_bytes, hipStream_t st) {
     using Cfg = StreamCfg<MT, TNW>;
     static std::once_flag once;
     static hipError_t e0 = hipSuccess, e1 = hipSuccess;
     std::call_once(once, [&] {
-        e0 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, false>, Cfg::kLds);
-        e1 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, true>, Cfg::kLds);
+        const int max_lds = Cfg::kLds + (XSL ? Cfg::scale_lds_bytes(Cfg::kMaxScaleSteps) : 0);
+        e0 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, false, XSL>, max_lds);
+        e1 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, true, XSL>, max_lds);
     });
     if (e0 != hipSuccess || e1 != hipSuccess) return MI355_ELAUNCH;
     if (pl.splits <= 1) {
-        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, false>), dim3(pl.tiles), dim3(256), Cfg::kLds, st, a);
+        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, false, XSL>), dim3(pl.tiles), dim3(256), lds_bytes, st,
+                           a);
     } else {
         a.splits = pl.splits;
         a.counters = (uint32_t *)ws;
         a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
-        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, true>), dim3(pl.tiles * pl.splits), dim3(256), Cfg::kLds,
-                           st, a);
+        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, true, XSL>), dim3(pl.tiles * pl.splits), dim3(256),
+                           lds_bytes, st, a);
     }
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+}
+
+// The activation scales of a CTA's K range are staged in LDS when the range is short enough for the staging area.
+template <int MT, int TNW>
+static int launch_stream(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStream_t st) {
+    using Cfg = StreamCfg<MT, TNW>;
+    const int KB = a.K / kBlockK;
+    const int steps = (KB + pl.splits - 1) / pl.splits;
+    if (steps <= Cfg::kMaxScaleSteps)
+        return launch_stream_as<MT, TNW, true>(a, pl, ws, Cfg::kLds + Cfg::scale_lds_bytes(steps), st);
+    return launch_stream_as<MT, TNW, false>(a, pl, ws, Cfg::kLds, st);
 }
 
 template <int MT>

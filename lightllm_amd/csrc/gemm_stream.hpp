@@ -2,7 +2,7 @@
 //
 // At these sizes the GEMM is a single pass over the N x K weight bytes, so the kernel is built around the
 // memory system, not the MFMA: every wave issues plain 16-byte-per-lane global loads in which 8 consecutive
-// lanes cover one 128-byte row segment (fully coalesced), keeps DEPTH K-steps of them in flight in registers,
+// lanes cover one 128-byte row segment (fully coalesced), keeps 1-3 K-steps of them in flight in registers,
 // and only then rearranges the bytes into MFMA operand order through a small wave-private LDS area
 // (ds_write_b128 / ds_read_b128, no workgroup barrier in the loop).  Loads that target LDS directly
 // (global_load_lds) sustain visibly less HBM bandwidth than plain loads on this part, which is why the
@@ -18,6 +18,10 @@
 //   through LDS; with cross-CTA splits the sum goes to the workspace and the last CTA to arrive adds the
 //   splits in order (deterministic) before the bf16 store.
 //
+// The activation scales of the CTA's K range are staged in LDS by one coalesced pass at the start: gathered per
+// step (16 rows x 4 bytes per request) they cost as many cache-line accesses as the X block itself, 5-6 us of a
+// 30-40 us launch at M = 32..64.
+//
 // Algorithmic bytes per K step and CTA: 16*TNW*128 weight bytes + 16*MT*128 activation bytes (L2 resident).
 #pragma once
 #include "gemm_tile.hpp"
@@ -30,28 +34,41 @@ template <int MT, int TNW>
 struct StreamCfg {
     static_assert(TNW == 1 || TNW == 2 || TNW == 4 || TNW == 8, "a tile must sit inside one 128-row scale block");
     static constexpr int BN = 16 * TNW;
-    static constexpr int kSetRegs = 8 * TNW + 9 * MT + 1;        // registers of one in-flight K step
-    static constexpr int kDepth = kSetRegs * 6 <= 150 ? 6 : (150 / kSetRegs < 2 ? 2 : 150 / kSetRegs);
+    // K steps in flight per wave.  Occupancy counts for more than depth: the deepest pipeline that still leaves a
+    // wave within 256 registers, i.e. two CTAs per CU (measured: M=32 28.9 us at depth 3 -> 25.6 at depth 2,
+    // M=64 36.6 us at depth 2 -> 33.9 at depth 1, M<=16 best at depth 3).
+    static constexpr int depth(bool xs_in_lds) {
+        if (xs_in_lds) return MT == 1 ? 3 : (MT == 2 ? 2 : 1);
+        const int set = 8 * TNW + 9 * MT + 1;  // registers of one in-flight K step
+        return set * 6 <= 150 ? 6 : (150 / set < 2 ? 2 : 150 / set);
+    }
     static constexpr int kXOff = 16 * TNW * 128;                  // X block follows the W block
     static constexpr int kWaveLds = (16 * TNW + 16 * MT) * 128;
     static constexpr int kAccLds = TNW * MT * 1024;               // one wave's accumulators (fp32)
     static constexpr int kWaveBytes = kWaveLds > kAccLds ? kWaveLds : kAccLds;
     static constexpr int kLds = kStreamWaves * kWaveBytes + 16;   // + the split-K arrival word
     static constexpr int kTileElems = 16 * MT * BN;
+    // activation scales of the CTA's K range, staged once: [step][16*MT rows + 1 pad] floats behind kLds
+    static constexpr int kScaleStride = 16 * MT + 1;
+    static constexpr int kMaxScaleSteps = 15 * 1024 / (kScaleStride * 4) < 64 ? 15 * 1024 / (kScaleStride * 4) : 64;
+    static constexpr int scale_lds_bytes(int steps) { return steps * kScaleStride * 4; }
 };
 
 template <int MT, int TNW>
 struct StreamRegs {
     v4i w[2 * TNW];  // 16*TNW rows x 128 B of W: instruction i holds rows 8i + lane/8, 16-byte chunk lane%8
     v4i x[2 * MT];   // 16*MT rows x 128 B of X, same arrangement
-    float xs[MT];    // activation scales of rows 16*mt + lane%16
+    float xs[MT];    // activation scales of rows 16*mt + lane%16 (unused when they are staged in LDS)
     float ws;        // weight scale of this (n block, K step)
 };
 
-template <int MT, int TNW, bool SPLIT>
+// XSL: the activation scales of the CTA's K range are staged in LDS by one coalesced pass at the start (the host
+// checks that the range fits); otherwise every wave gathers them per step, which costs as many cache-line
+// accesses as the X block itself (16 rows x 4 bytes per request).
+template <int MT, int TNW, bool SPLIT, bool XSL>
 __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmArgs p) {
     using Cfg = StreamCfg<MT, TNW>;
-    constexpr int D = Cfg::kDepth;
+    constexpr int D = Cfg::depth(XSL);
     constexpr int BN = Cfg::BN;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -92,6 +109,23 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
     const int NB = (p.N + kBlockN - 1) / kBlockN;
     const float *wsp = p.Ws + (int64_t)min(n0 / kBlockN, NB - 1) * p.ws_n;
 
+    // ---- stage the activation scales: thread (row group tid/32, step tid%32) walks rows +8 and steps +32, so a
+    // row-major scale row is read as whole cache lines; indices past the range repeat the last valid element
+    float *xs_lds = (float *)(lds + Cfg::kLds);
+    constexpr int kSvRows = 2 * MT, kSvSteps = (Cfg::kMaxScaleSteps + 31) / 32;
+    float sv[XSL ? kSvRows * kSvSteps : 1];
+    const int steps_cta = kb_end - kb_begin;
+    if constexpr (XSL) {
+#pragma unroll
+        for (int a = 0; a < kSvRows; ++a)
+#pragma unroll
+            for (int b = 0; b < kSvSteps; ++b) {
+                const int m = min(8 * a + (tid >> 5), p.M - 1);
+                const int kb = min(kb_begin + min(32 * b + (tid & 31), max(steps_cta - 1, 0)), KB - 1);
+                sv[a * kSvSteps + b] = p.Xs[(int64_t)m * p.xs_m + (int64_t)kb * p.xs_k];
+            }
+    }
+
     auto load = [&](StreamRegs<MT, TNW> &r, int kb) {
         const uint8_t *wk = p.W + (int64_t)kb * kBlockK;
         const uint8_t *xk = p.X + (int64_t)kb * kBlockK;
@@ -99,8 +133,10 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
         for (int i = 0; i < 2 * TNW; ++i) r.w[i] = __builtin_nontemporal_load((const v4i *)(wk + woff[i]));
 #pragma unroll
         for (int i = 0; i < 2 * MT; ++i) r.x[i] = *(const v4i *)(xk + xoff[i]);
+        if constexpr (!XSL) {
 #pragma unroll
-        for (int t = 0; t < MT; ++t) r.xs[t] = p.Xs[soff[t] + (int64_t)kb * p.xs_k];
+            for (int t = 0; t < MT; ++t) r.xs[t] = p.Xs[soff[t] + (int64_t)kb * p.xs_k];
+        }
         r.ws = wsp[(int64_t)kb * p.ws_k];
     };
 
@@ -132,7 +168,13 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
 #pragma unroll
         for (int j = 0; j < TNW; ++j) acc[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](const StreamRegs<MT, TNW> &r) {
+    auto consume = [&](const StreamRegs<MT, TNW> &r, int kb) {
+        float xsv[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            if constexpr (XSL) xsv[t] = xs_lds[(kb - kb_begin) * Cfg::kScaleStride + 16 * t + r16];
+            else xsv[t] = r.xs[t];
+        }
 #pragma unroll
         for (int i = 0; i < 2 * TNW; ++i) *(v4i *)(my + wst[i]) = r.w[i];
 #pragma unroll
@@ -150,7 +192,7 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
             const v4i lo = *(const v4i *)(my + Cfg::kXOff + rd0 + t * 2048);
             const v4i hi = *(const v4i *)(my + Cfg::kXOff + rd1 + t * 2048);
             const v8i xf = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            const float sc = r.xs[t] * r.ws;
+            const float sc = xsv[t] * r.ws;
 #pragma unroll
             for (int j = 0; j < TNW; ++j) {
                 const v4f part = mfma_16x16x128_fp8(wf[j], xf, v4f{0.f, 0.f, 0.f, 0.f});
@@ -164,11 +206,22 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
 #pragma unroll
     for (int d = 0; d < D; ++d)
         if (d < steps) load(regs[d], first + d * kStreamWaves);
+    if constexpr (XSL) {
+        // the scale loads were issued before the prologue loads, so only they are waited for here
+#pragma unroll
+        for (int a = 0; a < kSvRows; ++a)
+#pragma unroll
+            for (int b = 0; b < kSvSteps; ++b) {
+                const int j = 32 * b + (tid & 31);
+                if (j < steps_cta) xs_lds[j * Cfg::kScaleStride + 8 * a + (tid >> 5)] = sv[a * kSvSteps + b];
+            }
+        __syncthreads();
+    }
     for (int j = 0; j < steps; j += D) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             if (j + d < steps) {
-                consume(regs[d]);
+                consume(regs[d], first + (j + d) * kStreamWaves);
                 if (j + d + D < steps) load(regs[d], first + (j + d + D) * kStreamWaves);
             }
         }

@@ -204,6 +204,24 @@ def test_llama_decode_shapes(hip, M, N, K):
     _check_full(M, N, K, None, seed=M + 5)
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 16384, 8192), (8, 16384, 8448), (20, 1024, 4736), (33, 2048, 7168)])
+def test_stream_kernel_scale_staging(hip, M, N, K):
+    """The M <= 64 kernel stages the activation scales of a CTA's K range in LDS when the range is short enough
+    (59 steps at M > 32, else 64) and gathers them per step otherwise: both paths, an uneven K split (37 steps
+    over 2 CTAs) and a 56-step range just under the limit."""
+    print(f"gemm stream scale staging M={M} N={N} K={K}", flush=True)
+    _check_full(M, N, K, "skinny", seed=M + 3)
+
+
+def test_stream_kernel_column_major_scales(hip):
+    print("gemm stream column-major scales", flush=True)
+    xq, xs, wq, ws = _prep(24, 512, 2048, seed=77)
+    xs_cm = xs.t().contiguous().t()
+    C = _run(xq, xs_cm, wq, ws, "skinny")
+    _check_small(xq, xs, wq, ws, C)
+    assert torch.equal(C, _run(xq, xs, wq, ws, "skinny"))
+
+
 @pytest.mark.parametrize("N,K,variant", [(36864, 7168, "tile256"), (7168, 18432, None), (2112, 7168, None),
                                          (2112, 7168, "tile256"), (7168, 18432, "tile256x128")])
 def test_deepseek_prefill_shapes(hip, N, K, variant):
