@@ -89,7 +89,10 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
  * one (for tests and tuning).  Split-K variants need `ws` of at least
  * mi355_block_fp8_gemm_workspace_bytes() bytes, whose first MI355_WS_COUNTER_BYTES must be zero
  * on the first call; the kernels leave them zero again, so one zero-initialised buffer serves every call
- * issued in order on one stream.
+ * issued in order on one stream.  MI355_GEMM_TILE256 uses only those counter bytes and only if it gets them:
+ * with them the launch is persistent (one workgroup per compute unit takes tiles from per-XCD counters and
+ * overlaps the first requests of a tile with the stores of the previous one), without them (ws = NULL) every
+ * tile gets its own workgroup; same results.
  */
 #define MI355_GEMM_AUTO 0
 #define MI355_GEMM_TILE256 1     /* 256x256x128 CTA tile, 8 waves, LDS double buffer: compute-bound M */
@@ -124,7 +127,9 @@ int mi355_moe_align_fused(const int32_t *topk_ids, const float *topk_weights, in
 /* rows of the schedule table: min(num_pairs, ceil((num_pairs + E*(block_m-1)) / block_m))  (:457-458) */
 int64_t mi355_moe_align2_rows(int64_t num_pairs, int32_t num_experts, int32_t block_m);
 
-/* table int32 [rows,3] = (expert, m_index, token_start); padding rows get expert = -1 (:439-446). */
+/* table int32 [rows,4] = (expert, m_index, token_start, tokens in the block); padding rows get expert = -1
+ * (:439-446; the fourth column is derived, min(block_m, count - m_index*block_m), so that a GEMM tile needs one
+ * 16-byte load to know its work). */
 int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32_t block_m, int64_t rows,
                      int32_t *table, void *stream);
 
@@ -142,6 +147,11 @@ int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32
  * pairs in LightLLM's use); the masked expert-parallel layout passes a [E, T_pad] table with num_pairs = T_pad.
  * block_m must be one the library was built for: 16, 32, 64, 128, or 256 (256 needs K % 1024 == 0 and returns
  * MI355_EUNSUPPORTED otherwise); mi355_grouped_block_m() suggests one.
+ * workspace: optional, used by block_m = 256 only: MI355_WS_COUNTER_BYTES bytes that are zero before the launch
+ * (the kernel leaves them zero).  With it the launch is persistent - one workgroup per compute unit takes tiles
+ * from per-XCD counters and overlaps the first requests of a tile with the stores of the previous one;
+ * without it (NULL) every tile gets its own workgroup, same results.  Launches that may run concurrently
+ * need separate workspaces.
  */
 int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K);
 
@@ -150,7 +160,7 @@ int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W,
                                  const int32_t *expert_token_num, const int32_t *table, int64_t table_rows,
                                  int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
                                  int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
-                                 void *stream);
+                                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- element-wise steps between / after the two expert GEMMs ------------------------------------------------ */
 

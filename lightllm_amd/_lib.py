@@ -32,7 +32,8 @@ SIGNATURES = {
     "mi355_grouped_block_m": (_i32, [_i64, _i32, _i64, _i64]),
     "mi355_grouped_block_fp8_gemm": (
         _c.c_int,
-        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp],
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp,
+         _c.c_size_t, _vp],
     ),
     "mi355_silu_and_mul": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mi355_silu_and_mul_group_quant_fp8": (
@@ -96,7 +97,7 @@ _workspaces = {}
 
 
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Per (device, stream) scratch for split-K launches: zero-initialised once, grown on demand.
+    """Per (device, stream) scratch for split-K and persistent launches: zero-initialised once, grown on demand.
 
     The kernels leave the counter words zero, so the buffer is never cleared again.  Growing allocates, so
     callers that capture HIP graphs must run each shape once before capturing (as with any torch allocator use).

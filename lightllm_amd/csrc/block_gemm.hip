@@ -2,6 +2,7 @@
 #include <cstdlib>
 #include <mutex>
 
+#include "gemm_pp.hpp"
 #include "gemm_stream.hpp"
 #include "gemm_tile.hpp"
 
@@ -69,17 +70,38 @@ template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
 static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
     constexpr bool kFits = ((Cfg::lds_bytes(144) + 127) & ~127) + 2 * BM * 32 <= kMaxLds;  // up to K = 18432
-    if constexpr (MODE == kDensePP || MODE == kGroupedPP) {
-        return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
-    } else {
-        if constexpr (kFits) {
-            if (chunked_scales_ok(a)) {
-                const int r = launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
-                if (r != MI355_EUNSUPPORTED) return r;
-            }
+    if constexpr (kFits) {
+        if (chunked_scales_ok(a)) {
+            const int r = launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
+            if (r != MI355_EUNSUPPORTED) return r;
         }
-        return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false>(a, grid, st);
     }
+    return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false>(a, grid, st);
+}
+
+// The 256x256 ping-pong kernel.  a.tiles_m / a.tiles_n / a.total_tiles are set by the caller.  With a workspace
+// whose counter words are zero the launch is persistent (one workgroup per CU, tiles handed out per XCD);
+// without one every workgroup runs a single tile.  Returns MI355_EUNSUPPORTED when the K range does not fit
+// the kernel's LDS layout or the X scales cannot be fetched in chunks.
+template <bool GROUPED>
+static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hipStream_t st) {
+    if (!chunked_scales_ok(a)) return MI355_EUNSUPPORTED;
+    const int lds_bytes = PPCfg::lds_bytes(a.K / kBlockK);
+    if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
+    auto kernel = block_fp8_gemm_pp_kernel<GROUPED>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] { attr_err = allow_lds(kernel, kMaxLds); });
+    if (attr_err != hipSuccess) return MI355_ELAUNCH;
+    a.blocks_per_xcd = (a.total_tiles + 7) / 8;
+    int per_xcd = a.blocks_per_xcd;
+    a.counters = nullptr;
+    if (ws && ws_bytes >= (size_t)MI355_WS_COUNTER_BYTES && ((uintptr_t)ws & 3) == 0 && cus >= 8) {
+        a.counters = (uint32_t *)ws;
+        if (per_xcd > cus / 8) per_xcd = cus / 8;
+    }
+    hipLaunchKernelGGL(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_bytes, st, a);
+    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE = kDense>
@@ -212,6 +234,7 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
         const int splits = tile128_splits(M, N, K, 256);
         return splits > 1 ? tile128_workspace(M, N, splits) * 2 : 0;  // x2: headroom for devices with more CUs
     }
+    if (variant == MI355_GEMM_TILE256) return MI355_WS_COUNTER_BYTES;  // the tile counters of the persistent launch
     if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
     // sized for the deepest split (a one-CU device), so the figure does not depend on the device
     return skinny_workspace(M, skinny_plan(M, N, K, 1 << 20));
@@ -267,9 +290,17 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
     a.vec_store = (((uintptr_t)C & 15) == 0 && ldc % 8 == 0 && N % 8 == 0) ? 1 : 0;
 
     switch (variant) {
+        case 7:  // the ping-pong kernel with one workgroup per tile, workspace or not (kept for comparison)
+            ws = nullptr;
+            [[fallthrough]];
         case MI355_GEMM_TILE256: {
-            // the ping-pong kernel fetches X scales eight K steps at a time: row-major scales, 16-byte aligned rows
-            if (chunked_scales_ok(a)) return launch_dense<256, 256, 2, 4, 2, kDensePP>(a, st);
+            // the ping-pong kernel fetches X scales eight K steps at a time (row-major scales, 16-byte aligned
+            // rows); other layouts take the plain ring
+            a.tiles_m = (a.M + 255) / 256;
+            a.tiles_n = (a.N + 255) / 256;
+            a.total_tiles = a.tiles_m * a.tiles_n;
+            const int r = launch_pp<false>(a, ws, ws_bytes, cus, st);
+            if (r != MI355_EUNSUPPORTED) return r;
             return launch_dense<256, 256, 2, 4, 2>(a, st);
         }
         case 6:  // the plain ring kernel on the 256x256 tile, whatever the scale layout (kept for comparison)
@@ -324,7 +355,8 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
                                             const int32_t *expert_token_num, const int32_t *table,
                                             int64_t table_rows, int32_t block_m, int64_t num_pairs,
                                             int64_t num_tokens, int32_t num_experts, int32_t topk_num, int64_t N,
-                                            int64_t K, int32_t mul_routed_weight, void *out, void *stream) {
+                                            int64_t K, int32_t mul_routed_weight, void *out, void *ws,
+                                            size_t ws_bytes, void *stream) {
     if (num_pairs < 0 || num_tokens < 0 || num_experts <= 0 || topk_num <= 0 || N < 0 || K < 0 || table_rows < 0)
         return MI355_EINVAL;
     if (num_pairs == 0 || N == 0 || table_rows == 0) return MI355_OK;
@@ -379,8 +411,8 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
         case 64: return launch_tile<64, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
         case 128: return launch_tile<128, 128, 2, 2, 2, kGrouped>(a, finish(128), st);
         case 256:
-            if (!chunked_scales_ok(a)) return MI355_EUNSUPPORTED;
-            return launch_tile<256, 256, 2, 4, 2, kGroupedPP>(a, finish(256), st);
+            finish(256);
+            return launch_pp<true>(a, ws, ws_bytes, device_cus(), st);
         default: return MI355_EINVAL;
     }
 }

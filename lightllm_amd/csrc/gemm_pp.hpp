@@ -1,0 +1,445 @@
+// Block-scaled FP8 GEMM for gfx950: the 256x256 ping-pong kernel behind the large dense and grouped launches.
+//
+// Same arithmetic, LDS tile layout and epilogue as the ring kernel in gemm_tile.hpp (see there for the operand
+// layouts); what differs is the schedule:
+//
+//   * Two wave groups (waves 0-3 and 4-7: one wave of each per SIMD) run the phases of a K step
+//         A0  read the W fragments and the first half of the X fragments (+ their scales)
+//         B0  16 MFMA + scale folds of the first half
+//         A1  read the second half of the X fragments (+ scales)
+//         B1  16 MFMA + scale folds of the second half
+//     one phase apart, a barrier after each, so the MFMA bursts of one group overlap the LDS / DMA traffic of the
+//     other.  Group 1 passes one extra barrier before its first phase and group 0 one after its last.
+//   * Two ring slots of { X 256 x 128 B, W 256 x 128 B }.  A region of a slot is requested again as soon as both
+//     groups have read it: the W rows and first-half X rows of step it+2 at A1(it), the second-half X rows of
+//     step it+1 at A0(it).  Every request is waited for one and a half steps later, by every wave, before the
+//     barrier that lets the first group read it.  The loop body has no branches in the dense launch (steps past
+//     the end re-fetch the last step, identical bytes) so the phases stay where they are written.
+//   * X scales come in [256 rows][8 steps] chunks (one 16-byte request per half row and chunk, two buffers):
+//     one column per step would cost as many cache-line requests as the X tile itself.
+//   * The kernel is persistent: a workgroup keeps taking tiles, and between two tiles it issues the first
+//     requests of the next tile before it stores the finished one, so the request latency, the stores and the
+//     index gathers of the grouped launch overlap.  A fresh workgroup per tile costs about 9 us of such
+//     serialized latencies per tile (10 % of a 56-step tile, 25 % of a 16-step one).
+//     Tiles are numbered per XCD (workgroup ids go round-robin over the 8 XCDs): sequence number v on XCD x is
+//     logical tile x*blocks_per_xcd + v of the dense order (runs of 8 m tiles x all n, so the tiles that share
+//     an L2 share panels) or tile 8*v + x of the grouped launch order (n fastest: tiles differ in cost and the
+//     schedule table is padded at its end, so they are dealt out).  The first two sequence numbers of a
+//     workgroup are static (its index in the XCD, + workgroups per XCD), later ones come from one atomic counter
+//     per XCD in the caller's workspace, fetched two tiles ahead; the schedule-table row of a tile is loaded one
+//     tile ahead.  Counter words: [0..7] per-XCD, [8] workgroups that have finished; the last one to finish
+//     zeroes them again.  Without a workspace (counters == nullptr) every workgroup runs one tile.
+#pragma once
+#include "gemm_tile.hpp"
+
+namespace mi355 {
+
+struct PPCfg {
+    static constexpr int BM = 256, BN = 256, kWaves = 8, kThreads = 512;
+    static constexpr int WMS = 128, WNS = 64;   // a wave's sub-tile: 2 x 4 waves
+    static constexpr int TM = 8, TN = 4, HM = 4;
+    static constexpr int XI = 4, WI = 4;         // 8-row DMA groups per wave: 32 of X and 32 of W over 8 waves
+    static constexpr int kStage = (BM + BN) * 128;
+    static constexpr int kDummyOff = 2 * kStage;     // 256-byte target of place-holder requests
+    static constexpr int kWsOff = kDummyOff + 256;   // two buffers of the tile's weight scales [2 n blocks][KB]
+    static constexpr int kChunkBytes = BM * 32;      // one [256 rows][8 steps] chunk of X scales
+    static constexpr int ws_bytes(int KB) { return 2 * KB * 4; }
+    static constexpr int chunk_off(int KB) { return (kWsOff + 2 * ws_bytes(KB) + 127) & ~127; }
+    static constexpr int sched_off(int KB) { return chunk_off(KB) + 2 * kChunkBytes; }
+    static constexpr int lds_bytes(int KB) { return sched_off(KB) + 16; }
+    static constexpr int kCounterWords = 9;
+};
+
+template <bool GROUPED>
+__global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p) {
+    using Cfg = PPCfg;
+    constexpr int BM = Cfg::BM, TM = Cfg::TM, TN = Cfg::TN, HM = Cfg::HM, WMS = Cfg::WMS, WNS = Cfg::WNS;
+    constexpr bool SKIP = GROUPED;  // ragged tiles skip empty halves; dense tiles keep the branch-free body
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 2, wave_n = wave & 3;
+    const int grp = wave >> 2;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const int sub = lane >> 3;
+    const uint32_t pch = (uint32_t)(lane & 7);
+    const int KB = p.K / kBlockK, nk = KB, nchunk = KB >> 3;
+    const uint32_t lds0 = lds_addr(lds);
+    const uint32_t xcd = blockIdx.x & 7u, in_xcd = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+    const bool persistent = p.counters != nullptr;
+    volatile uint32_t *sched = (volatile uint32_t *)(lds + Cfg::sched_off(KB));
+    constexpr uint32_t kNone = 0xffffffffu;
+
+    // ---- tile-independent LDS offsets
+    uint32_t xdst[Cfg::XI], wdst[Cfg::WI];
+#pragma unroll
+    for (int i = 0; i < Cfg::XI; ++i) xdst[i] = (uint32_t)(wave + i * Cfg::kWaves) * 1024u;
+#pragma unroll
+    for (int i = 0; i < Cfg::WI; ++i) wdst[i] = (uint32_t)BM * 128u + (uint32_t)(wave + i * Cfg::kWaves) * 1024u;
+    const uint32_t fr = swz((uint32_t)r16);
+    const uint32_t c0 = ((uint32_t)(2 * g4)) ^ fr, c1 = c0 ^ 1u;
+    const uint32_t xrow = (uint32_t)(wave_m * WMS + r16) * 128u;
+    const uint32_t wrow = (uint32_t)BM * 128u + (uint32_t)(wave_n * WNS + r16) * 128u;
+    const uint32_t xr0 = xrow + c0 * 16u, xr1 = xrow + c1 * 16u;
+    const uint32_t wr0 = wrow + c0 * 16u, wr1 = wrow + c1 * 16u;
+    const uint32_t chunk_off = (uint32_t)Cfg::chunk_off(KB);
+    const uint32_t sr8 = chunk_off + (uint32_t)(wave_m * WMS + r16) * 32u;
+
+    // ---- the tile a sequence number names
+    struct Tile {
+        int m0;      // dense: first row; grouped: first slot of the expert's list
+        int n0;
+        int rows;    // valid rows
+        int expert;
+        bool valid;
+    };
+    auto tile_coords = [&](uint32_t v, uint32_t &tile_m, uint32_t &tile_n) -> bool {
+        if (v == kNone) return false;
+        if constexpr (GROUPED) {
+            const uint64_t bid = (uint64_t)v * 8u + xcd;
+            if (bid >= (uint64_t)p.total_tiles) return false;
+            tile_m = (uint32_t)bid / (uint32_t)p.tiles_n;
+            tile_n = (uint32_t)bid - tile_m * (uint32_t)p.tiles_n;
+        } else {
+            if (v >= (uint32_t)p.blocks_per_xcd) return false;
+            const uint32_t logical = xcd * (uint32_t)p.blocks_per_xcd + v;
+            if (logical >= (uint32_t)p.total_tiles) return false;
+            constexpr uint32_t GM = 8;
+            const uint32_t width = GM * (uint32_t)p.tiles_n;
+            const uint32_t g = logical / width;
+            const uint32_t first_m = g * GM;
+            const uint32_t gsz = min((uint32_t)p.tiles_m - first_m, GM);
+            const uint32_t in_grp = logical - g * width;
+            tile_m = first_m + in_grp % gsz;
+            tile_n = in_grp / gsz;
+        }
+        return true;
+    };
+    // grouped: the schedule-table row (expert, m_index, token_start, rows) of sequence number v; expert < 0 = none
+    auto load_row = [&](uint32_t v) -> v4i {
+        uint32_t tm = 0, tn = 0;
+        if (!GROUPED || !tile_coords(v, tm, tn)) return v4i{-1, 0, 0, 0};
+        return *(const v4i *)(p.table + (int64_t)tm * 4);
+    };
+    auto make_tile = [&](uint32_t v, v4i row) -> Tile {
+        Tile t = {0, 0, 0, 0, false};
+        uint32_t tm = 0, tn = 0;
+        if (!tile_coords(v, tm, tn)) return t;
+        t.n0 = (int)tn * Cfg::BN;
+        if constexpr (GROUPED) {
+            t.expert = __builtin_amdgcn_readfirstlane(row[0]);
+            if (t.expert < 0) return t;
+            t.m0 = __builtin_amdgcn_readfirstlane(row[1]) * BM;
+            t.rows = __builtin_amdgcn_readfirstlane(row[3]);
+        } else {
+            t.m0 = (int)tm * BM;
+            t.rows = min(p.M - t.m0, BM);
+        }
+        t.m0 = __builtin_amdgcn_readfirstlane(t.m0);
+        t.n0 = __builtin_amdgcn_readfirstlane(t.n0);
+        t.rows = __builtin_amdgcn_readfirstlane(t.rows);
+        t.valid = true;
+        return t;
+    };
+
+    // ---- per-tile request state
+    uint32_t xoff[Cfg::XI], woff[Cfg::WI], sc_off = 0;
+    bool x_real[Cfg::XI];
+    bool do_half0 = true, do_half1 = true;
+    const uint8_t *xg = p.X, *wg = p.W;
+    const float *sg = p.Xs;
+    int wsbuf = 0;  // weight-scale buffer of the tile in the K loop
+
+    // row gathers of a tile (grouped): slot -> token row.  Issued early, used by finish_setup.
+    auto gather = [&](const Tile &t, uint32_t (&raw)[Cfg::XI + 1]) {
+        if constexpr (GROUPED) {
+            const int32_t *idx_list = p.e2t_index + (int64_t)t.expert * p.num_pairs + t.m0;
+#pragma unroll
+            for (int i = 0; i < Cfg::XI; ++i) raw[i] = (uint32_t)idx_list[min((wave + i * Cfg::kWaves) * 8 + sub, t.rows - 1)];
+            raw[Cfg::XI] = (uint32_t)idx_list[min(wave * 32 + (lane >> 1), t.rows - 1)];
+        } else {
+#pragma unroll
+            for (int i = 0; i < Cfg::XI; ++i) raw[i] = (uint32_t)min((wave + i * Cfg::kWaves) * 8 + sub, t.rows - 1);
+            raw[Cfg::XI] = (uint32_t)min(wave * 32 + (lane >> 1), t.rows - 1);
+        }
+    };
+    const uint8_t *w_tile = p.W;   // W rows of the tile (expert and n0 applied)
+    const float *ws_tile = p.Ws;   // weight scales of the tile's expert
+    auto setup_w = [&](const Tile &t) {
+        w_tile = p.W + (GROUPED ? (int64_t)t.expert * p.w_e : (int64_t)0) + (int64_t)t.n0 * p.ldw;
+        ws_tile = p.Ws + (GROUPED ? (int64_t)t.expert * p.ws_e : (int64_t)0);
+        wg = w_tile;
+#pragma unroll
+        for (int i = 0; i < Cfg::WI; ++i) {
+            const int rho = (wave + i * Cfg::kWaves) * 8 + sub;  // LDS row
+            const uint32_t c = pch ^ swz((uint32_t)rho);
+            const int span = rho / WNS, w = rho % WNS;
+            const int tn = w >> 4, gg = (w >> 2) & 3, vv = w & 3;
+            const int nl = span * WNS + lane_col<TN>(gg, tn) + vv;
+            const int nc = min(t.n0 + nl, p.N - 1) - t.n0;
+            woff[i] = (uint32_t)nc * (uint32_t)p.ldw + c * 16u;
+        }
+    };
+    auto setup_x = [&](const Tile &t, const uint32_t (&raw)[Cfg::XI + 1]) {
+        xg = p.X + (GROUPED ? (int64_t)0 : (int64_t)t.m0 * p.ldx);
+        sg = p.Xs + (GROUPED ? (int64_t)0 : (int64_t)t.m0 * p.xs_m);
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; ++i) {
+            const int r = (wave + i * Cfg::kWaves) * 8 + sub;
+            const uint32_t c = pch ^ swz((uint32_t)r);
+            const uint32_t src_row = GROUPED ? raw[i] / (uint32_t)p.topk : raw[i];
+            xoff[i] = src_row * (uint32_t)p.ldx + c * 16u;
+            x_real[i] = !SKIP || (wave + i * Cfg::kWaves) * 8 < t.rows;
+        }
+        const uint32_t srow = GROUPED ? raw[Cfg::XI] / (uint32_t)p.topk : raw[Cfg::XI];
+        sc_off = (srow * (uint32_t)p.xs_m + 4u * (uint32_t)(lane & 1)) * 4u;
+        do_half0 = !SKIP || wave_m * WMS < t.rows;
+        do_half1 = !SKIP || wave_m * WMS + WMS / 2 < t.rows;
+    };
+    // the tile's weight scales (2 n blocks x all K steps) go to LDS buffer `buf` in two parts: the load is issued
+    // with the tile's first requests, the LDS write waits until the stores of the previous tile are out (a
+    // write right behind the load would wait for every request issued before it)
+    auto ws_elem = [&](const Tile &t, int i) -> float {
+        const int NB = (p.N + kBlockN - 1) / kBlockN;
+        const int b = i / KB, kb = i - b * KB;
+        const int nb = min(t.n0 / kBlockN + b, NB - 1);
+        return ws_tile[(int64_t)nb * p.ws_n + (int64_t)kb * p.ws_k];
+    };
+    auto ws_load = [&](const Tile &t) -> float { return tid < 2 * KB ? ws_elem(t, tid) : 0.f; };
+    auto ws_store = [&](const Tile &t, int buf, float first) {
+        float *wl = (float *)(lds + Cfg::kWsOff + buf * Cfg::ws_bytes(KB));
+        if (tid < 2 * KB) wl[tid] = first;
+        for (int i = tid + Cfg::kThreads; i < 2 * KB; i += Cfg::kThreads) wl[i] = ws_elem(t, i);  // K > 32768 only
+    };
+
+    // ---- DMA requests.  An 8-row X group past the last valid row of a ragged tile is not fetched; a one-line
+    // request takes its place so that every wave counts the same number of requests.
+    auto issue_x = [&](int i, uint32_t sb, const uint8_t *xk) {
+        if (x_real[i]) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+        else dma_g2l_b32(lds0 + Cfg::kDummyOff, p.X, 0u);
+    };
+    auto issue_w = [&](int stage, int kb) {
+        const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
+        const uint8_t *wk = wg + (int64_t)kb * kBlockK;
+#pragma unroll
+        for (int i = 0; i < Cfg::WI; ++i) dma_g2l_b128(sb + wdst[i], wk, woff[i]);
+    };
+    auto issue_xlo = [&](int stage, int kb) {
+        const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
+        const uint8_t *xk = xg + (int64_t)kb * kBlockK;
+#pragma unroll
+        for (int i = 0; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
+    };
+    auto issue_xhi = [&](int stage, int kb) {
+        const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
+        const uint8_t *xk = xg + (int64_t)kb * kBlockK;
+#pragma unroll
+        for (int i = 1; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
+    };
+    // lane l of wave w fetches steps 4*(l&1).. of row 32*w + l/2 of the chunk: scale (row, kb) then sits at
+    // chunk[(kb/8) & 1][row][kb % 8]
+    auto issue_scales = [&](int chunk) {
+        dma_g2l_b128(lds0 + chunk_off + (uint32_t)(chunk & 1) * Cfg::kChunkBytes + (uint32_t)wave * 1024u, sg + 8 * chunk, sc_off);
+    };
+    constexpr int kXhi = Cfg::XI / 2;             // requests per wave in A0
+    constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;  // requests per wave in A1
+
+    auto phase_end = [&]() {
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler only: no LDS access may move across the barrier
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+    };
+    auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8)); };
+
+    // ---- start: the first tile and the row of the second
+    uint32_t v_next = persistent ? per_xcd + in_xcd : kNone;  // sequence number of the tile after the current one
+    uint32_t v_after = kNone;                                 // and of the one after that (fetched)
+    uint32_t fetched = 0;
+    Tile cur = make_tile(in_xcd, load_row(in_xcd));
+    v4i row_next = load_row(v_next);
+    if (persistent && tid == 0)
+        fetched = __hip_atomic_fetch_add(p.counters + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (cur.valid) {
+        uint32_t raw[Cfg::XI + 1];
+        gather(cur, raw);
+        setup_w(cur);
+        issue_w(0, 0);
+        issue_w(1, min(1, nk - 1));
+        setup_x(cur, raw);
+        issue_scales(0);
+        issue_xlo(0, 0);
+        issue_xhi(0, 0);
+        issue_xlo(1, min(1, nk - 1));
+        ws_store(cur, 0, ws_load(cur));
+    }
+    wait_vmcnt<0>();
+    if (persistent && tid == 0) sched[0] = 2u * per_xcd + fetched;
+    __syncthreads();
+    if (persistent) v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
+
+    v4f acc[TM][TN];
+    while (cur.valid) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        const float *wsl = (const float *)(lds + Cfg::kWsOff + wsbuf * Cfg::ws_bytes(KB)) + ((wave_n * WNS) / kBlockN) * KB;
+
+        // ---- the K loop
+        if (grp == 1) phase_end();
+        int slot = 0;
+        for (int it = 0; it < nk; ++it) {
+            const uint8_t *st = lds + slot * Cfg::kStage;
+            const int cbuf = (it >> 3) & 1;
+            // A0 (LDS reads first: a DMA request can stall the wave's issue, the reads behind it would wait)
+            const float ws_cur = wsl[it];
+            const float *sp = (const float *)(lds + sr8 + cbuf * Cfg::kChunkBytes + (it & 7) * 4);
+            v8i wf[TN], xf[HM];
+            if (do_half0) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
+                    const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
+                    wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const bool do_half = h == 0 ? do_half0 : do_half1;
+                float xs[HM];
+                if (do_half) {
+#pragma unroll
+                    for (int i = 0; i < HM; ++i) {
+                        const v4i lo = *(const v4i *)(st + xr0 + (h * HM + i) * 2048);
+                        const v4i hi = *(const v4i *)(st + xr1 + (h * HM + i) * 2048);
+                        xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        xs[i] = sp[(h * HM + i) * 16 * 8] * ws_cur;
+                    }
+                }
+                if (h == 0) {
+                    if ((it & 7) == 0 && (it >> 3) + 1 < nchunk) issue_scales((it >> 3) + 1);
+                    issue_xhi(slot ^ 1, min(it + 1, nk - 1));
+                } else {
+                    issue_xlo(slot, min(it + 2, nk - 1));
+                    issue_w(slot, min(it + 2, nk - 1));
+                }
+                // everything but the last two request groups has landed: at the end of A0 that covers the second
+                // X half of this step, at the end of A1 the W rows and first X half of the next one (the scale
+                // request of every eighth step only makes the wait one request stricter)
+                wait_vmcnt<kXhi + kWXlo>();
+                wait_lds();
+                phase_end();
+                // B0 / B1: the scale fold of a product is issued kLag MFMAs after its own MFMA, when the result
+                // has long left the matrix pipe (a fold right behind the next MFMA would cost 7 idle issue
+                // slots every other product)
+                if (do_half) {
+                    constexpr int E = HM * TN, kLag = 2;
+                    v4f parts[kLag + 1];
+#pragma unroll
+                    for (int e = 0; e < E + kLag; ++e) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (e < E) parts[e % (kLag + 1)] = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
+                        if (e >= kLag) {
+                            const int f = e - kLag;
+                            acc[h * HM + f / TN][f % TN] += parts[f % (kLag + 1)] * xs[f / TN];
+                        }
+                        if (e < E && e >= kLag) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
+                            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // an older product's fold behind it
+                        }
+                    }
+                }
+                phase_end();
+            }
+            slot ^= 1;
+        }
+        if (grp == 0) phase_end();
+        wait_vmcnt<0>();  // the re-fetches of the last steps have landed: the slots are free
+
+        // ---- between two tiles: first requests of the next tile, then the stores of this one
+        const Tile done = cur;
+        float ws_first = 0.f;
+        cur = make_tile(v_next, row_next);
+        if (cur.valid) {
+            uint32_t raw[Cfg::XI + 1];
+            gather(cur, raw);
+            setup_w(cur);
+            issue_w(0, 0);
+            issue_w(1, min(1, nk - 1));
+            // sequence number and table row for later tiles (used one and two tiles from now)
+            v_next = v_after;
+            row_next = load_row(v_next);
+            if (persistent && tid == 0)
+                fetched = __hip_atomic_fetch_add(p.counters + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            wsbuf ^= 1;
+            ws_first = ws_load(cur);
+            setup_x(cur, raw);
+            issue_scales(0);
+            issue_xlo(0, 0);
+            issue_xhi(0, 0);
+            issue_xlo(1, min(1, nk - 1));
+        }
+
+        // epilogue of the finished tile: lane (r16, g4) holds, for each tm, row wave_m*WMS + 16*tm + r16 and, for
+        // each block pair h, the 8 columns n0 + wave_n*WNS + lane_col(g4, 2h) + [0, 8)
+        {
+            const int nbase = done.n0 + wave_n * WNS;
+            const int32_t *idx_list = GROUPED ? p.e2t_index + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
+            const float *w_list = GROUPED ? p.e2t_weight + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int rl = wave_m * WMS + 16 * i + r16;
+                if (rl >= done.rows) continue;
+                int64_t out_row;
+                float rw = 1.0f;
+                if constexpr (GROUPED) {
+                    out_row = idx_list[rl];
+                    if (p.mul_weight) rw = w_list[rl];
+                } else {
+                    out_row = done.m0 + rl;
+                }
+                uint16_t *cp = p.C + out_row * p.ldc + nbase;
+                float o[4 * TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = GROUPED ? acc[i][j][vv] * rw : acc[i][j][vv];
+                if (p.vec_store && nbase + WNS <= p.N) {
+#pragma unroll
+                    for (int h = 0; h < TN / 2; ++h)
+                        *(v4i *)(cp + lane_col<TN>(g4, 2 * h)) =
+                            v4i{(int)pack_bf16x2(o[8 * h + 0], o[8 * h + 1]), (int)pack_bf16x2(o[8 * h + 2], o[8 * h + 3]),
+                                (int)pack_bf16x2(o[8 * h + 4], o[8 * h + 5]), (int)pack_bf16x2(o[8 * h + 6], o[8 * h + 7])};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4 * TN; ++e) {
+                        const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
+                        if (nbase + c < p.N) cp[c] = (uint16_t)f32_to_bf16_bits(o[e]);
+                    }
+                }
+            }
+        }
+        wait_vmcnt<0>();
+        if (cur.valid) {
+            ws_store(cur, wsbuf, ws_first);
+            if (persistent && tid == 0) sched[0] = 2u * per_xcd + fetched;
+            __syncthreads();
+            if (persistent) v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
+        }
+    }
+
+    // ---- the last workgroup to finish leaves the counters zero for the next launch
+    if (persistent && tid == 0) {
+        const uint32_t prev = __hip_atomic_fetch_add(p.counters + 8, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (prev == gridDim.x - 1) {
+#pragma unroll
+            for (int i = 0; i < Cfg::kCounterWords; ++i)
+                __hip_atomic_store(p.counters + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+}  // namespace mi355

@@ -18,15 +18,14 @@
 //   n block), then - with chunked scales - two [BM rows][8 steps] buffers of X scales.
 //   Rows are 128 B = 8 chunks of 16 B, chunk position XOR-swizzled with the row number (swz() in common.hpp)
 //   so the ds_read_b128 operand fetches are conflict free.  W rows are stored in the order the MFMA wants
-//   them: LDS row 16*tn + 4*g + v of a wave span holds weight row 4*TN*g + 4*tn + v, which makes every lane's
-//   4*TN outputs contiguous in n (one or two 16-byte stores).  Tiles are filled with global_load_lds_dwordx4
+//   them: LDS row 16*tn + 4*g + v of a wave span holds weight row lane_col<TN>(g, tn) + v, which makes the
+//   16-byte stores of the four lane groups of a token row adjacent (see lane_col).  Tiles are filled with global_load_lds_dwordx4
 //   (no register staging); each 8-lane group fetches one full 128-byte row segment.
 //
 // Pipelines
-//   ring       NSTAGE stages; the DMA for step kb+NSTAGE-1 is issued at the top of step kb, right after the
-//              one barrier of the step (which also proves that the slot being refilled has been read by all).
-//   ping-pong  the 256x256 tile only: two wave groups run LDS phases and MFMA phases one phase apart, ring
-//              slot regions are refilled as soon as both groups have read them (see the kernel body).
+//   A ring of NSTAGE stages; the DMA for step kb+NSTAGE-1 is issued at the top of step kb, right after the one
+//   barrier of the step (which also proves that the slot being refilled has been read by all).  The large
+//   256x256 launches use the ping-pong kernel in gemm_pp.hpp instead.
 //
 // Launch modes
 //   kDense     one CTA per output tile, whole K, ring.
@@ -35,13 +34,12 @@
 //              partials in split order (deterministic), writes bf16 and re-zeroes the counter.
 //   kGrouped   rows are gathered through expert_to_token_index, the tile list is the moe_align2 table, the
 //              weight and its scales are offset by the expert, rows are scattered back on store.
-//   kDensePP / kGroupedPP   the dense and the grouped launch on the ping-pong pipeline.
 #pragma once
 #include "common.hpp"
 
 namespace mi355 {
 
-enum { kDense = 0, kGrouped = 1, kSplitK = 2, kDensePP = 3, kGroupedPP = 4 };
+enum { kDense = 0, kGrouped = 1, kSplitK = 2 };
 
 struct GemmArgs {
     const uint8_t *X;    // [M,K] (dense) or [T,K] (grouped), row stride ldx bytes
@@ -59,13 +57,25 @@ struct GemmArgs {
     uint32_t *counters;  // [total_tiles], zero before the launch, zero again after it
     float *partials;     // [total_tiles][splits][BM*BN]
     // grouped launch only
-    const int32_t *table;        // [tiles_m,3] (expert, m_index, token_start)
+    const int32_t *table;        // [tiles_m,4] (expert, m_index, token_start, rows)
     const int32_t *e2t_index;    // [E,num_pairs]
     const float *e2t_weight;     // [E,num_pairs]
     const int32_t *e_num;        // [E]
     int64_t w_e, ws_e;           // expert strides of W (bytes) and Ws (elements)
     int32_t num_pairs, topk, mul_weight;
 };
+
+// Which of a wave's 16*TN output columns a lane holds.  The MFMA leaves lane group g (= lane / 16) with the four
+// results v = 0..3 of A-operand rows 4*g + v of each of the TN 16-row blocks; which weight row sits in which
+// A-operand row is free (it is fixed when the W tile is laid out in LDS).  The choice below makes the 8 values
+// of a block pair (2h, 2h+1) eight consecutive columns, and the four lane groups of one token row adjacent
+// 16-byte pieces: one store instruction then writes 64 contiguous bytes per row.  (With 16 consecutive columns
+// per lane the pieces of one instruction were 32 bytes apart, and the L2 took four times as many write
+// requests: 6 us per 256x256 tile.)
+template <int TN>
+__device__ __forceinline__ constexpr int lane_col(int g, int tn) {
+    return TN == 1 ? 4 * g : 32 * (tn >> 1) + 8 * g + 4 * (tn & 1);
+}
 
 template <int BM, int BN, int WM, int WN, int NSTAGE>
 struct TileCfg {
@@ -99,11 +109,9 @@ struct TileCfg {
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
 __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const GemmArgs p) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
-    constexpr bool PINGPONG = MODE == kDensePP || MODE == kGroupedPP;
-    static_assert(!PINGPONG || XS8, "the ping-pong schedule needs chunked scales");
     constexpr int kLoads = Cfg::XI + Cfg::WI + (XS8 ? 0 : 1);  // DMA requests per wave and stage
     constexpr int TM = Cfg::TM, TN = Cfg::TN, WMS = Cfg::WMS, WNS = Cfg::WNS;
-    constexpr bool GROUPED = MODE == kGrouped || MODE == kGroupedPP;
+    constexpr bool GROUPED = MODE == kGrouped;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     // ---- which tile (and which K range)
@@ -114,7 +122,7 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         split = blockIdx.x - tile_id * (uint32_t)p.splits;
         tile_m = tile_id % (uint32_t)p.tiles_m;
         tile_n = tile_id / (uint32_t)p.tiles_m;
-    } else if constexpr (MODE == kGrouped || MODE == kGroupedPP) {
+    } else if constexpr (MODE == kGrouped) {
         // The schedule table is padded with empty rows at its end and tiles differ in cost, so tiles are dealt
         // out in launch order, n fastest: the n tiles of one m block land on different XCDs, and (tiles_n being
         // a multiple of 8 for the usual shapes) the same weight tile of consecutive m blocks on the same XCD.
@@ -155,9 +163,9 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     const float *Wsbase = p.Ws;
     int rows_valid;  // number of valid rows in this tile
     if constexpr (GROUPED) {
-        const int expert = p.table[tile_m * 3 + 0];
+        const int expert = p.table[tile_m * 4 + 0];
         if (expert < 0) return;
-        const int mi = p.table[tile_m * 3 + 1];
+        const int mi = p.table[tile_m * 4 + 1];
         const int cnt = p.e_num[expert];
         m0 = mi * BM;
         idx_list = p.e2t_index + (int64_t)expert * p.num_pairs;
@@ -193,7 +201,7 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         const uint32_t c = pch ^ swz((uint32_t)rho);
         const int span = rho / WNS, w = rho % WNS;
         const int tn = w >> 4, gg = (w >> 2) & 3, v = w & 3;
-        const int nl = span * WNS + 4 * TN * gg + 4 * tn + v;
+        const int nl = span * WNS + lane_col<TN>(gg, tn) + v;
         const int nc = min(n0 + nl, p.N - 1) - n0;
         woff[i] = (uint32_t)nc * (uint32_t)p.ldw + c * 16u;
         wdst[i] = (uint32_t)BM * 128u + (uint32_t)grpi * 1024u;
@@ -296,205 +304,64 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     }
     const int nk = kb_end - kb_begin;
 
-    if constexpr (PINGPONG) {
-        // Two-group ping-pong with early refill, for the 256x256 tile (8 waves, two ring slots).
-        //
-        // The 8 waves form two groups (waves 0-3 and 4-7: one wave of each group per SIMD) that run the same
-        // phase sequence one phase apart, so while one group's waves keep the matrix pipe busy the other
-        // group's waves fetch operands from LDS and feed the DMA.  Phases of one K step, a barrier after each:
-        //   A0  read the W fragments and the first half of the X fragments (+ their scales)
-        //   B0  MFMA + scale fold of the first half
-        //   A1  read the second half of the X fragments (+ scales)
-        //   B1  MFMA + scale fold of the second half
-        // Group 1 starts one barrier late and group 0 ends one barrier late, so both count the same number.
-        //
-        // The pipeline is bound by the L2 -> LDS path, so a region of a ring slot is refilled as soon as both
-        // groups have read it instead of once per step: the W rows and the first-half X rows of tile it+2 are
-        // requested at the top of A1(it) (into the slot tile it is leaving), the second-half X rows of tile
-        // it+1 at the top of A0(it).  Every request is waited for one and a half steps later, by every wave,
-        // before the barrier that lets the first group read it.  The loop body has no branches (steps past the
-        // end re-fetch the last tile, identical bytes) so that the phases stay where they are written.
-        //
-        // The X scales come in [256 rows][8 steps] chunks (see issue_scales), requested in the first step of
-        // the previous chunk.
-        static_assert(NSTAGE == 2 && Cfg::kWaves == 8 && TM % 2 == 0 && Cfg::XI == 4 && BM == 256, "ping-pong layout");
-        constexpr int HM = TM / 2;
-        // Ragged (grouped) tiles: a wave whose 64-row half holds no valid row skips that half's LDS reads and
-        // MFMAs (never the barriers or the DMA requests, which every wave must count alike).  Dense tiles keep
-        // the branch-free body.
-        constexpr bool SKIP = GROUPED;
-        const bool do_half0 = !SKIP || wave_m * WMS < rows_valid;
-        const bool do_half1 = !SKIP || wave_m * WMS + WMS / 2 < rows_valid;
-        constexpr int kXhi = Cfg::XI / 2;              // requests per wave in A0 (X second half)
-        constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;   // requests per wave in A1
-        const int grp = wave >> 2;
-        auto phase_end = [&]() {
-            __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler only: no LDS access may move across the barrier
-            __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_barrier();
-            __builtin_amdgcn_sched_barrier(0);
-            __atomic_signal_fence(__ATOMIC_SEQ_CST);
-        };
-        auto wait_lds = [&]() { __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8)); };
-        // Ragged tiles: an 8-row X group past the last valid row is not fetched.  Every wave must still count
-        // the same number of requests, so a one-line request (all lanes read the first 4 bytes of X into a spare
-        // LDS area) takes its place.
-        bool x_real[Cfg::XI];
+    // prologue: the scale chunk of the first step and the one after it, then NSTAGE-1 stages
+    if constexpr (XS8) {
+        issue_scales(kb_begin >> 3);
+        if ((kb_begin >> 3) + 1 < nchunk) issue_scales((kb_begin >> 3) + 1);
+    }
 #pragma unroll
-        for (int i = 0; i < Cfg::XI; ++i) x_real[i] = !SKIP || ((wave + i * Cfg::kWaves) % Cfg::XG) * 8 < rows_valid;
-        auto issue_x = [&](int i, uint32_t sb, const uint8_t *xk) {
-            if (x_real[i]) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
-            else dma_g2l_b32(lds0 + Cfg::kScaleOff, p.X, 0u);
-        };
-        auto issue_wxlo = [&](int stage, int kb) {
-            const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
-            const uint8_t *xk = xg + (int64_t)kb * kBlockK;
-            const uint8_t *wk = wg + (int64_t)kb * kBlockK;
-#pragma unroll
-            for (int i = 0; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
-#pragma unroll
-            for (int i = 0; i < Cfg::WI; ++i) dma_g2l_b128(sb + wdst[i], wk, woff[i]);
-        };
-        auto issue_xhi = [&](int stage, int kb) {
-            const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
-            const uint8_t *xk = xg + (int64_t)kb * kBlockK;
-#pragma unroll
-            for (int i = 1; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
-        };
-        issue_scales(0);
-        issue_wxlo(0, 0);
-        issue_xhi(0, 0);
-        issue_wxlo(1, min(1, nk - 1));
-        wait_vmcnt<kWXlo>();
+    for (int s = 0; s < NSTAGE - 1; ++s)
+        if (s < nk) issue(s, kb_begin + s);
+
+    int cur = 0;            // ring slot of step it
+    int fill = NSTAGE - 1;  // ring slot the next DMA goes to
+    for (int it = 0; it < nk; ++it) {
+        // stage `it` must have landed; the NSTAGE-2 stages issued after it may still be in flight
+        // (a scale-chunk request in between only makes the wait stricter: requests retire in order)
+        if (it + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * kLoads>();
+        else wait_vmcnt<0>();
         __syncthreads();
-        if (grp == 1) phase_end();
-        int cur = 0;
-        for (int it = 0; it < nk; ++it) {
-            const uint8_t *st = lds + cur * Cfg::kStage;
-            const int cbuf = (it >> 3) & 1;
-            // ---- A0 (LDS reads first: a DMA request can stall the wave's issue, the reads behind it would wait)
-            const float ws_cur = wsl[it];
-            const float *sp = (const float *)(lds + sr8 + cbuf * kChunkBytes + (it & 7) * 4);
-            v8i wf[TN], xf[HM];
-            if (do_half0) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
-                    const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
-                    wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                }
-            }
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const bool do_half = h == 0 ? do_half0 : do_half1;
-                float xs[HM];
-                if (do_half) {
-#pragma unroll
-                    for (int i = 0; i < HM; ++i) {
-                        const v4i lo = *(const v4i *)(st + xr0 + (h * HM + i) * 2048);
-                        const v4i hi = *(const v4i *)(st + xr1 + (h * HM + i) * 2048);
-                        xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        xs[i] = sp[(h * HM + i) * 16 * 8] * ws_cur;
-                    }
-                }
-                if (h == 0) {
-                    if ((it & 7) == 0 && (it >> 3) + 1 < nchunk) issue_scales((it >> 3) + 1);
-                    issue_xhi(cur ^ 1, min(it + 1, nk - 1));
-                } else {
-                    issue_wxlo(cur, min(it + 2, nk - 1));
-                }
-                // everything but the last two request groups has landed: at the end of A0 that covers the second
-                // X half of this tile, at the end of A1 the W rows and first X half of the next one (the scale
-                // request of every eighth step only makes the wait one request stricter)
-                wait_vmcnt<kXhi + kWXlo>();
-                wait_lds();
-                phase_end();
-                // ---- B0 / B1: the scale fold of a product is issued kLag MFMAs after its own MFMA, when the
-                // result has long left the matrix pipe (a fold right behind the next MFMA would cost 7 idle
-                // issue slots every other product)
-                if (do_half) {
-                    constexpr int E = HM * TN, kLag = 2;
-                    v4f parts[kLag + 1];
-#pragma unroll
-                    for (int e = 0; e < E + kLag; ++e) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (e < E) parts[e % (kLag + 1)] = mfma_16x16x128_fp8(wf[e % TN], xf[e / TN], v4f{0.f, 0.f, 0.f, 0.f});
-                        if (e >= kLag) {
-                            const int f = e - kLag;
-                            acc[h * HM + f / TN][f % TN] += parts[f % (kLag + 1)] * xs[f / TN];
-                        }
-                        if (e < E && e >= kLag) {
-                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // the MFMA first,
-                            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // an older product's fold behind it
-                        }
-                    }
-                }
-                phase_end();
-            }
-            cur ^= 1;
-        }
-        if (grp == 0) phase_end();
-        wait_vmcnt<0>();  // the re-fetches of the last steps must not outlive the workgroup's LDS
-    } else {
-        // prologue: the scale chunk of the first step and the one after it, then NSTAGE-1 stages
+        const int kb = kb_begin + it;
         if constexpr (XS8) {
-            issue_scales(kb_begin >> 3);
-            if ((kb_begin >> 3) + 1 < nchunk) issue_scales((kb_begin >> 3) + 1);
+            // the buffer of chunk kb/8 + 1 was last read in step kb - 1, before the barrier above
+            if ((kb & 7) == 0 && it > 0 && (kb >> 3) + 1 < nchunk) issue_scales((kb >> 3) + 1);
+        }
+        if (it + NSTAGE - 1 < nk) issue(fill, kb_begin + it + NSTAGE - 1);
+        const float ws_cur = wsl[kb_begin + it];
+
+        const uint8_t *st = lds + cur * Cfg::kStage;
+        float xs[TM];
+        if constexpr (XS8) {
+            const float *sp = (const float *)(lds + sr8 + ((kb >> 3) & 1) * kChunkBytes + (kb & 7) * 4);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) xs[i] = sp[i * 16 * 8] * ws_cur;
+        } else {
+            const float *sp = (const float *)(lds + sr + cur * (BM * 4));
+#pragma unroll
+            for (int i = 0; i < TM; ++i) xs[i] = sp[i] * ws_cur;
+        }
+        v8i wf[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
+            const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
+            wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         }
 #pragma unroll
-        for (int s = 0; s < NSTAGE - 1; ++s)
-            if (s < nk) issue(s, kb_begin + s);
-
-        int cur = 0;            // ring slot of step it
-        int fill = NSTAGE - 1;  // ring slot the next DMA goes to
-        for (int it = 0; it < nk; ++it) {
-            // stage `it` must have landed; the NSTAGE-2 stages issued after it may still be in flight
-            // (a scale-chunk request in between only makes the wait stricter: requests retire in order)
-            if (it + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * kLoads>();
-            else wait_vmcnt<0>();
-            __syncthreads();
-            const int kb = kb_begin + it;
-            if constexpr (XS8) {
-                // the buffer of chunk kb/8 + 1 was last read in step kb - 1, before the barrier above
-                if ((kb & 7) == 0 && it > 0 && (kb >> 3) + 1 < nchunk) issue_scales((kb >> 3) + 1);
-            }
-            if (it + NSTAGE - 1 < nk) issue(fill, kb_begin + it + NSTAGE - 1);
-            const float ws_cur = wsl[kb_begin + it];
-
-            const uint8_t *st = lds + cur * Cfg::kStage;
-            float xs[TM];
-            if constexpr (XS8) {
-                const float *sp = (const float *)(lds + sr8 + ((kb >> 3) & 1) * kChunkBytes + (kb & 7) * 4);
-#pragma unroll
-                for (int i = 0; i < TM; ++i) xs[i] = sp[i * 16 * 8] * ws_cur;
-            } else {
-                const float *sp = (const float *)(lds + sr + cur * (BM * 4));
-#pragma unroll
-                for (int i = 0; i < TM; ++i) xs[i] = sp[i] * ws_cur;
-            }
-            v8i wf[TN];
+        for (int i = 0; i < TM; ++i) {
+            const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
+            const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
+            const v8i xf = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
-                const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
-                wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const v4f part = mfma_16x16x128_fp8(wf[j], xf, v4f{0.f, 0.f, 0.f, 0.f});
+                acc[i][j] += part * xs[i];
             }
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
-                const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
-                const v8i xf = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    const v4f part = mfma_16x16x128_fp8(wf[j], xf, v4f{0.f, 0.f, 0.f, 0.f});
-                    acc[i][j] += part * xs[i];
-                }
-            }
-            cur = cur + 1 == NSTAGE ? 0 : cur + 1;
-            fill = fill + 1 == NSTAGE ? 0 : fill + 1;
         }
-
+        cur = cur + 1 == NSTAGE ? 0 : cur + 1;
+        fill = fill + 1 == NSTAGE ? 0 : fill + 1;
     }
+
 
     // ---- split-K: publish the partial, let the last CTA of the tile reduce
     // Partials and the arrival counter are exchanged with agent-scope relaxed atomics: such stores write
@@ -538,9 +405,9 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         if (tid == 0) __hip_atomic_store(p.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    // ---- epilogue: lane (r16, g4) holds, for each tm, row m = wave_m*WMS + 16*tm + r16 and the 4*TN
-    // consecutive columns n = n0 + wave_n*WNS + 4*TN*g4 + [0, 4*TN).
-    const int ncol = n0 + wave_n * WNS + 4 * TN * g4;
+    // ---- epilogue: lane (r16, g4) holds, for each tm, row m = wave_m*WMS + 16*tm + r16 and, for each MFMA block
+    // tn, the 4 columns n0 + wave_n*WNS + lane_col(g4, tn) + [0, 4).
+    const int nbase = n0 + wave_n * WNS;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int rl = wave_m * WMS + 16 * i + r16;
@@ -553,26 +420,28 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
         } else {
             out_row = m0 + rl;
         }
-        uint16_t *cp = p.C + out_row * p.ldc + ncol;
+        uint16_t *cp = p.C + out_row * p.ldc + nbase;
         float o[4 * TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[4 * j + v] = GROUPED ? acc[i][j][v] * rw : acc[i][j][v];
-        if (p.vec_store && ncol + 4 * TN <= p.N) {
+        if (p.vec_store && nbase + WNS <= p.N) {
             if constexpr (TN == 1) {
-                *(v2i *)cp = v2i{(int)pack_bf16x2(o[0], o[1]), (int)pack_bf16x2(o[2], o[3])};
+                *(v2i *)(cp + lane_col<TN>(g4, 0)) = v2i{(int)pack_bf16x2(o[0], o[1]), (int)pack_bf16x2(o[2], o[3])};
             } else {
 #pragma unroll
                 for (int h = 0; h < TN / 2; ++h)
-                    *(v4i *)(cp + 8 * h) =
+                    *(v4i *)(cp + lane_col<TN>(g4, 2 * h)) =
                         v4i{(int)pack_bf16x2(o[8 * h + 0], o[8 * h + 1]), (int)pack_bf16x2(o[8 * h + 2], o[8 * h + 3]),
                             (int)pack_bf16x2(o[8 * h + 4], o[8 * h + 5]), (int)pack_bf16x2(o[8 * h + 6], o[8 * h + 7])};
             }
         } else {
 #pragma unroll
-            for (int e = 0; e < 4 * TN; ++e)
-                if (ncol + e < p.N) cp[e] = (uint16_t)f32_to_bf16_bits(o[e]);
+            for (int e = 0; e < 4 * TN; ++e) {
+                const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
+                if (nbase + c < p.N) cp[c] = (uint16_t)f32_to_bf16_bits(o[e]);
+            }
         }
     }
 }

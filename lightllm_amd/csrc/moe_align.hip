@@ -82,13 +82,14 @@ __global__ __launch_bounds__(256) void moe_align2_kernel(const int32_t *__restri
     for (int b = tid; b < nblk; b += 256) {
         const int64_t r = (int64_t)block_start + b;
         if (r < rows) {
-            table[r * 3 + 0] = expert;
-            table[r * 3 + 1] = b;
-            table[r * 3 + 2] = token_start + b * block_m;
+            table[r * 4 + 0] = expert;
+            table[r * 4 + 1] = b;
+            table[r * 4 + 2] = token_start + b * block_m;
+            table[r * 4 + 3] = min(cnt - b * block_m, block_m);
         }
     }
     if (expert == num_experts - 1)
-        for (int64_t r = (int64_t)block_start + nblk + tid; r < rows; r += 256) table[r * 3 + 0] = -1;
+        for (int64_t r = (int64_t)block_start + nblk + tid; r < rows; r += 256) table[r * 4 + 0] = -1;
 }
 
 }  // namespace mi355

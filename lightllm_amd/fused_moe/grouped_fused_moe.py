@@ -44,14 +44,15 @@ def moe_align_fused(expert_to_token_index, expert_to_weight, expert_token_num, t
 
 
 def moe_align2(token_num_mul_topk_num: int, exports_token_num: torch.Tensor, block_m: int):
-    """Expert counts [E] -> schedule table int32 [max_blocks, 3] of (expert, m_index, token_start);
+    """Expert counts [E] -> schedule table int32 [max_blocks, 4] of (expert, m_index, token_start,
+    tokens in the block);
     rows past the last real block have expert = -1."""
     assert exports_token_num.dtype == torch.int32 and exports_token_num.is_contiguous()
     _lib.require_cuda(exports_token_num)
     E = exports_token_num.shape[0]
     lib = _lib.lib()
     rows = lib.mi355_moe_align2_rows(token_num_mul_topk_num, E, block_m)
-    table = torch.empty((rows, 3), dtype=torch.int32, device=exports_token_num.device)
+    table = torch.empty((rows, 4), dtype=torch.int32, device=exports_token_num.device)
     code = lib.mi355_moe_align2(
         exports_token_num.data_ptr(), E, block_m, rows, table.data_ptr(), _lib.stream_ptr(table.device)
     )
@@ -124,12 +125,14 @@ def grouped_matmul(
     else:
         table = moe_align2(token_num_mul_topk_num, expert_to_token_num, block_m)
 
+    # the 256-row launch is persistent when it gets the (zero at rest) tile counters of this stream's workspace
+    ws = _lib.workspace(out.device, _lib.WS_COUNTER_BYTES) if block_m == 256 else None
     code = lib.mi355_grouped_block_fp8_gemm(
         token_inputs.data_ptr(), token_input_scale.data_ptr(), expert_weights.data_ptr(),
         expert_to_weights_scale.data_ptr(), expert_to_token_index.data_ptr(), expert_to_weights.data_ptr(),
         expert_to_token_num.data_ptr(), table.data_ptr(), table.shape[0], block_m, token_num_mul_topk_num,
         token_inputs.shape[0], expert_num, topk_num, n, k, 1 if mul_routed_weight else 0, out.data_ptr(),
-        _lib.stream_ptr(out.device),
+        ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _lib.stream_ptr(out.device),
     )
     _lib.check(code, "grouped_matmul")
     return (table, block_m)

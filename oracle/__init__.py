@@ -155,11 +155,11 @@ def moe_align_fused(topk_ids, topk_weights, num_experts: int):
 
 
 def moe_align2(num_pairs: int, expert_token_num, block_m: int) -> np.ndarray:
-    """-> int32 [max_blocks, 3]; columns 1,2 of padding rows are left at -1 here."""
+    """-> int32 [max_blocks, 4]; columns 1-3 of padding rows are left at -1 here."""
     cnt = _c(expert_token_num, np.int32)
     E = cnt.size
     rows = lib().oracle_moe_align2_rows(I64(num_pairs), I32(E), I32(block_m))
-    table = np.full((rows, 3), -1, np.int32)
+    table = np.full((rows, 4), -1, np.int32)
     lib().oracle_moe_align2(_p(cnt), I32(E), I32(block_m), I64(rows), _p(table))
     return table
 

@@ -275,25 +275,27 @@ int64_t oracle_moe_align2_rows(int64_t num_pairs, int32_t num_experts, int32_t b
 
 /*
  * moe_align2 (grouped_fused_moe.py:399-477): expand per-expert counts into the
- * schedule table of (expert, m_index, token_start) rows, one per block of
- * block_m tokens, experts in ascending order; rows past the last real block
- * get expert = -1 (only column 0 is written for them).
+ * schedule table of (expert, m_index, token_start, rows) rows, one per block
+ * of block_m tokens, experts in ascending order (`rows` = tokens in the block,
+ * derived: min(block_m, count - m_index*block_m)); rows past the last real
+ * block get expert = -1 (only column 0 is written for them).
  */
 void oracle_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32_t block_m,
-                       int64_t max_blocks, int32_t *table /* [max_blocks,3] */) {
+                       int64_t max_blocks, int32_t *table /* [max_blocks,4] */) {
     int64_t row = 0;
     int32_t token_start = 0;
     for (int32_t e = 0; e < num_experts; ++e) {
         int32_t cnt = expert_token_num[e];
         int32_t nblk = (cnt + block_m - 1) / block_m;
         for (int32_t b = 0; b < nblk && row < max_blocks; ++b, ++row) {
-            table[row * 3 + 0] = e;
-            table[row * 3 + 1] = b;
-            table[row * 3 + 2] = token_start + b * block_m;
+            table[row * 4 + 0] = e;
+            table[row * 4 + 1] = b;
+            table[row * 4 + 2] = token_start + b * block_m;
+            table[row * 4 + 3] = cnt - b * block_m < block_m ? cnt - b * block_m : block_m;
         }
         token_start += cnt;
     }
-    for (; row < max_blocks; ++row) table[row * 3 + 0] = -1;
+    for (; row < max_blocks; ++row) table[row * 4 + 0] = -1;
 }
 
 /*

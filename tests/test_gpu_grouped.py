@@ -63,6 +63,7 @@ def test_moe_align2_reference_vectors(hip):
     assert t[:, 0].tolist() == [0, 2, 2, 2, 2, 3, -1, -1, -1, -1]
     assert t[:6, 1].tolist() == [0, 0, 1, 2, 3, 0]
     assert t[:6, 2].tolist() == [0, 8, 24, 40, 56, 68]
+    assert t[:6, 3].tolist() == [8, 16, 16, 16, 12, 16]      # tokens per block (derived column)
     cnt = torch.zeros((10,), dtype=torch.int32, device="cuda")
     cnt[0] = 8
     t = moe_align2(8, cnt, block_m=16).cpu()

@@ -248,6 +248,7 @@ def test_moe_align2_reference_golden():
     assert t[:, 0].tolist() == [0, 2, 2, 2, 2, 3, -1, -1, -1, -1]
     assert t[:6, 1].tolist() == [0, 0, 1, 2, 3, 0]
     assert t[:6, 2].tolist() == [0, 8, 24, 40, 56, 68]
+    assert t[:6, 3].tolist() == [8, 16, 16, 16, 12, 16]
     t = oracle.moe_align2(8, [8] + [0] * 9, 16)
     assert t.shape[0] == 8 and t[0, 0] == 0 and np.all(t[1:, 0] == -1)
 
