@@ -91,6 +91,25 @@ def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
         _check_small(xq, xs, wq, ws, c_pp)
 
 
+def test_persistent_launch_matches_one_workgroup_per_tile(hip):
+    """With the workspace counters the ping-pong kernel is persistent (one workgroup per CU; from the third tile
+    on a workgroup takes tiles from per-XCD atomic counters), without them every tile gets its own workgroup.
+    1024 tiles: same bits either way, on repeated launches, and the counter words are zero again afterwards."""
+    from lightllm_amd import _lib
+
+    print("gemm persistent vs per-tile launch", flush=True)
+    M, N, K = 4096, 16384, 1024
+    xq, xs, wq, ws = _prep(M, N, K, seed=12)
+    once = _run(xq, xs, wq, ws, "tile256once").clone()
+    for _ in range(3):
+        assert torch.equal(_run(xq, xs, wq, ws, "tile256").view(torch.int16), once.view(torch.int16))
+    counters = _lib.workspace(xq.device, _lib.WS_COUNTER_BYTES)[:64]
+    assert int(counters.to(torch.int32).sum()) == 0 and not bool(counters.any())
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(once.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+
+
 def test_pingpong_tile_random_shapes(hip):
     """Twenty seeded random shapes (ragged M and N edges, several K): ping-pong and ring tiles agree bit for bit,
     and a sample of entries agrees with the float64 oracle."""

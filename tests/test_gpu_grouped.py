@@ -112,6 +112,50 @@ def test_grouped_256_row_blocks_vs_oracle(hip, mul_w, topk, T, E):
     _grouped_case(T=T, E=E, topk=topk, N=640, K=2048, block_m=256, mul_w=mul_w, seed=75)
 
 
+def test_grouped_persistent_launch_matches_one_workgroup_per_tile(hip, monkeypatch):
+    """The 256-row launch with the workspace counters (persistent, tiles handed out per XCD) against the same
+    kernel without a workspace (one workgroup per tile): about 600 tiles of mixed cost, identical bits, counter
+    words zero afterwards.  A sample of rows is checked against the torch fp32 dequant-matmul of its expert."""
+    from lightllm_amd import _lib
+    from lightllm_amd.fused_moe import grouped_matmul
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print("grouped persistent vs per-tile launch", flush=True)
+    T, E, topk, N, K = 2048, 24, 4, 4096, 1024
+    ids, tw = H.routing(T, E, topk, seed=95)
+    idx, w, cnt = _align(ids, tw, E)
+    x = H.activations(T, K, seed=96).cuda()
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, N // 128, K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=100 + e, device="cuda")
+    P = T * topk
+
+    def run():
+        out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        grouped_matmul(P, xq, xs, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=False, use_fp8_w8a8=True,
+                       run_config={"BLOCK_SIZE_M": 256})
+        torch.cuda.synchronize()
+        return out
+
+    persistent = [run() for _ in range(2)]
+    counters = _lib.workspace(xq.device, _lib.WS_COUNTER_BYTES)[:64]
+    assert not bool(counters.any())
+    with monkeypatch.context() as mp:
+        mp.setattr(_lib, "workspace", lambda *a, **k: None)
+        once = run()
+    assert not torch.isnan(once.float()).any()
+    for out in persistent:
+        assert torch.equal(out.view(torch.int16), once.view(torch.int16))
+    cnt_h, idx_h = cnt.cpu(), idx.cpu()
+    for e in range(0, E, 5):
+        pairs = idx_h[e, : int(cnt_h[e])].long()[:64].cuda()
+        ref = tr.dequant_matmul(xq[pairs // topk], xs[pairs // topk], wq[e], ws[e], out_dtype=torch.float32)
+        cos, rel = H.gemm_metrics(once[pairs].float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (e, cos, rel)
+
+
 def test_grouped_empty_and_single_token_experts(hip):
     """More experts than tokens: most experts get no rows, some one row; N tail (200 % 128 != 0)."""
     print("grouped sparse experts", flush=True)
