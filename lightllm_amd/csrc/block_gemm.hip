@@ -96,9 +96,10 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hipStream_
     a.blocks_per_xcd = (a.total_tiles + 7) / 8;
     int per_xcd = a.blocks_per_xcd;
     a.counters = nullptr;
-    if (ws && ws_bytes >= (size_t)MI355_WS_COUNTER_BYTES && ((uintptr_t)ws & 3) == 0 && cus >= 8) {
+    // persistent only when there is more than one tile per CU (a single round gains nothing from the tile queue)
+    if (ws && ws_bytes >= (size_t)MI355_WS_COUNTER_BYTES && ((uintptr_t)ws & 3) == 0 && per_xcd > cus / 8 && cus >= 8) {
         a.counters = (uint32_t *)ws;
-        if (per_xcd > cus / 8) per_xcd = cus / 8;
+        per_xcd = cus / 8;
     }
     hipLaunchKernelGGL(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_bytes, st, a);
     return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
@@ -290,7 +291,7 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
     a.vec_store = (((uintptr_t)C & 15) == 0 && ldc % 8 == 0 && N % 8 == 0) ? 1 : 0;
 
     switch (variant) {
-        case 7:  // the ping-pong kernel with one workgroup per tile, workspace or not (kept for comparison)
+        case MI355_GEMM_TILE256_ONCE:  // kept for comparison
             ws = nullptr;
             [[fallthrough]];
         case MI355_GEMM_TILE256: {
@@ -303,7 +304,7 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
             if (r != MI355_EUNSUPPORTED) return r;
             return launch_dense<256, 256, 2, 4, 2>(a, st);
         }
-        case 6:  // the plain ring kernel on the 256x256 tile, whatever the scale layout (kept for comparison)
+        case MI355_GEMM_TILE256_RING:  // kept for comparison
             return launch_dense<256, 256, 2, 4, 2>(a, st);
         case MI355_GEMM_TILE256x128:
             return launch_dense<256, 128, 2, 4, 3>(a, st);

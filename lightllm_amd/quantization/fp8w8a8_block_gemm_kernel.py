@@ -13,7 +13,7 @@ from .. import _lib
 _VARIANTS = {
     None: _lib.GEMM_AUTO, "auto": _lib.GEMM_AUTO, "tile256": _lib.GEMM_TILE256, "tile128": _lib.GEMM_TILE128,
     "skinny": _lib.GEMM_SKINNY, "generic": _lib.GEMM_GENERIC, "tile256x128": _lib.GEMM_TILE256x128,
-    "tile256ring": 6, "tile256once": 7,
+    "tile256ring": _lib.GEMM_TILE256_RING, "tile256once": _lib.GEMM_TILE256_ONCE,
 }
 
 
