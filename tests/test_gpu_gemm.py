@@ -91,14 +91,15 @@ def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
         _check_small(xq, xs, wq, ws, c_pp)
 
 
-def test_persistent_launch_matches_one_workgroup_per_tile(hip):
+@pytest.mark.parametrize("M,N,K", [(4096, 16384, 1024), (4000, 16400, 1024), (1100, 16385, 1024)])
+def test_persistent_launch_matches_one_workgroup_per_tile(hip, M, N, K):
     """With the workspace counters the ping-pong kernel is persistent (one workgroup per CU; from the third tile
     on a workgroup takes tiles from per-XCD atomic counters), without them every tile gets its own workgroup.
-    1024 tiles: same bits either way, on repeated launches, and the counter words are zero again afterwards."""
+    About 1000 tiles (and fewer, with ragged M and N edges and an N that forces element-wise stores): same bits
+    either way, on repeated launches, and the counter words are zero again afterwards."""
     from lightllm_amd import _lib
 
-    print("gemm persistent vs per-tile launch", flush=True)
-    M, N, K = 4096, 16384, 1024
+    print(f"gemm persistent vs per-tile launch M={M} N={N} K={K}", flush=True)
     xq, xs, wq, ws = _prep(M, N, K, seed=12)
     once = _run(xq, xs, wq, ws, "tile256once").clone()
     for _ in range(3):
