@@ -132,6 +132,33 @@ def test_pingpong_tile_random_shapes(hip):
         assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
 
 
+def test_stream_kernel_random_shapes(hip):
+    """Twenty-four seeded random decode-size shapes (every M class, N with and without a 64-row tail or a
+    vector-store-friendly width, K from one to 72 steps so that single-CTA and split-K launches, staged and
+    gathered scales all occur): the whole matrix against the torch fp32 dequant-matmul and a sample against the
+    float64 oracle; the slow generic kernel must agree within one bf16 ulp of the row scale."""
+    rng = np.random.default_rng(4711)
+    for case in range(24):
+        M = int(rng.choice([1, 2, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64]))
+        N = int(rng.integers(1, 400)) * int(rng.choice([1, 8, 16]))
+        K = int(rng.choice([128, 256, 1024, 2048, 4096, 7168, 9216]))
+        print(f"gemm stream random case {case}: M={M} N={N} K={K}", flush=True)
+        xq, xs, wq, ws = _prep(M, N, K, seed=3000 + case, device="cuda")
+        c = _run(xq, xs, wq, ws, "skinny")
+        assert not torch.isnan(c.float()).any()
+        ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+        cos, rel = H.gemm_metrics(c.float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (M, N, K, cos, rel)
+        g = _run(xq, xs, wq, ws, "generic")
+        assert (c.float() - g.float()).abs().max() <= ref.abs().max() * 2 ** -7, (M, N, K)
+        rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 4)])
+        cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 30)])
+        ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                              ws.cpu().numpy(), np.arange(len(rows)), cols)
+        got = c[rows][:, cols].float().cpu().double().numpy()
+        assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
+
+
 def test_unit_scales_is_plain_matmul(hip):
     """All scales 1: the result is the plain product of the fp8 values, exact in fp32 for K=128."""
     print("gemm unit scales", flush=True)

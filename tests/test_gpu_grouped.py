@@ -156,6 +156,51 @@ def test_grouped_persistent_launch_matches_one_workgroup_per_tile(hip, monkeypat
         assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (e, cos, rel)
 
 
+def test_grouped_random_shapes(hip):
+    """Sixteen seeded random routed batches (tokens, experts, top-k, N with a tail, K with and without chunked
+    scale fetches, every row-block size that the shape allows, routed weight on and off): every routed row against
+    the torch fp32 dequant-matmul of its expert."""
+    from lightllm_amd.fused_moe import grouped_matmul
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    rng = np.random.default_rng(97)
+    for case in range(16):
+        T = int(rng.integers(1, 700))
+        E = int(rng.integers(1, 20))
+        topk = int(rng.integers(1, min(E, 4) + 1))
+        N = int(rng.integers(1, 12)) * 64 + int(rng.choice([0, 8, 40]))
+        K = int(rng.choice([128, 384, 1024, 2048]))
+        blocks = [16, 32, 64, 128] + ([256] if K % 1024 == 0 else [])
+        block_m = int(rng.choice(blocks))
+        mul_w = bool(rng.integers(0, 2)) and topk == 1
+        print(f"grouped random case {case}: T={T} E={E} topk={topk} N={N} K={K} block_m={block_m} mul_w={mul_w}", flush=True)
+        ids, tw = H.routing(T, E, topk, seed=500 + case)
+        idx, w, cnt = _align(ids, tw, E)
+        x = H.activations(T, K, seed=600 + case).cuda()
+        xq, xs = per_token_group_quant_fp8(x, 128)
+        wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+        ws = torch.empty((E, -(-N // 128), K // 128), dtype=torch.float32, device="cuda")
+        for e in range(E):
+            wq[e], ws[e] = H.quantized_weights(N, K, seed=700 + 31 * case + e, device="cuda")
+        P = T * topk
+        out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        grouped_matmul(P, xq, xs, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=mul_w, use_fp8_w8a8=True,
+                       run_config={"BLOCK_SIZE_M": block_m})
+        torch.cuda.synchronize()
+        assert not torch.isnan(out.float()).any(), "a routed row was not written"
+        cnt_h, idx_h, w_h = cnt.cpu(), idx.cpu(), w.cpu()
+        for e in range(E):
+            n_e = int(cnt_h[e])
+            if n_e == 0:
+                continue
+            pairs = idx_h[e, :n_e].long().cuda()
+            ref = tr.dequant_matmul(xq[pairs // topk], xs[pairs // topk], wq[e], ws[e], out_dtype=torch.float32)
+            if mul_w:
+                ref = ref * w_h[e, :n_e].cuda()[:, None]
+            cos, rel = H.gemm_metrics(out[pairs].float(), ref)
+            assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (case, e, cos, rel)
+
+
 def test_grouped_empty_and_single_token_experts(hip):
     """More experts than tokens: most experts get no rows, some one row; N tail (200 % 128 != 0)."""
     print("grouped sparse experts", flush=True)
