@@ -203,7 +203,8 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 static int pick_variant(int64_t M, int64_t N, int cus) {
     if (M <= 64) return MI355_GEMM_SKINNY;
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (t256 >= (int64_t)cus / 2) return MI355_GEMM_TILE256;
+    // measured crossover (N=7168, K=18432): 56 tiles of 256x256 lose to split-K 128x128 tiles, 112 tiles win
+    if (t256 >= (int64_t)cus * 3 / 8) return MI355_GEMM_TILE256;
     return MI355_GEMM_TILE128;
 }
 
