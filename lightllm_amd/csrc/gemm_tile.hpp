@@ -19,8 +19,8 @@
 //   Rows are 128 B = 8 chunks of 16 B, chunk position XOR-swizzled with the row number (swz() in common.hpp)
 //   so the ds_read_b128 operand fetches are conflict free.  W rows are stored in the order the MFMA wants
 //   them: LDS row 16*tn + 4*g + v of a wave span holds weight row lane_col<TN>(g, tn) + v, which makes the
-//   16-byte stores of the four lane groups of a token row adjacent (see lane_col).  Tiles are filled with global_load_lds_dwordx4
-//   (no register staging); each 8-lane group fetches one full 128-byte row segment.
+//   16-byte stores of the four lane groups of a token row adjacent (see lane_col).  Tiles are filled with
+//   global_load_lds_dwordx4 (no register staging); each 8-lane group fetches one full 128-byte row segment.
 //
 // Pipelines
 //   A ring of NSTAGE stages; the DMA for step kb+NSTAGE-1 is issued at the top of step kb, right after the one

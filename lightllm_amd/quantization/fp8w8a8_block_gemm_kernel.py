@@ -35,7 +35,8 @@ def w8a8_block_fp8_matmul(
 
     A [M,K] e4m3fn contiguous; B [K,N] e4m3fn (LightLLM passes ``weight.t()``: strides (1,K));
     Ascale [M, K/128] fp32; Bscale [K/128, ceil(N/128)] fp32; C [M,N] bf16 contiguous.
-    ``run_config`` may be ``{"variant": "auto"|"tile256"|"tile256x128"|"tile128"|"skinny"|"generic"}``; the
+    ``run_config`` may be ``{"variant": "auto"|"tile256"|"tile256x128"|"tile128"|"skinny"|"generic"}`` (plus the
+    comparison variants "tile256ring" and "tile256once"); the
     reference's tile dictionaries (BLOCK_M, ...) are accepted and ignored: the shape table is built in.
     """
     assert len(block_size) == 2
