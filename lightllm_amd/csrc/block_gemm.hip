@@ -114,9 +114,9 @@ static int launch_dense(GemmArgs &a, hipStream_t st) {
     return launch_tile<BM, BN, WM, WN, NSTAGE, MODE>(a, a.blocks_per_xcd * 8, st);
 }
 
-// Weight-streaming launch for M <= 64: 64-row tiles (16-, 32- and 128-row tiles all measured slower on the
-// decode shapes), the K range split over CTAs only as far as needed to give every CU a CTA, and never below
-// 16 K steps per CTA (4 per wave).
+// Weight-streaming launch for M <= 64: 64-row tiles (32-row ones in the case below; 16- and 128-row tiles measured
+// slower on the decode shapes), the K range split over CTAs only as far as needed to give every CU a CTA, and
+// never below 16 K steps per CTA (4 per wave).
 static int skinny_mt(int64_t M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 
 struct SkinnyPlan {
@@ -124,9 +124,10 @@ struct SkinnyPlan {
 };
 
 static SkinnyPlan skinny_plan(int64_t M, int64_t N, int64_t K, int cus) {
-    (void)M;
     SkinnyPlan pl;
-    pl.tnw = 4;
+    // 32-row tiles when 64-row ones are fewer than the CUs and M > 16 (N=4096, K=14336: 17.7 / 22.5 us at M=32 / 64
+    // against 19.6 / 24.6; no difference at M <= 16, and slower when N alone fills the device)
+    pl.tnw = (M > 16 && (N + 63) / 64 < cus) ? 2 : 4;
     pl.tiles = (int)((N + 16 * pl.tnw - 1) / (16 * pl.tnw));
     const int KB = (int)(K / kBlockK);
     pl.splits = (cus + pl.tiles - 1) / pl.tiles;
@@ -179,6 +180,7 @@ template <int MT>
 static int launch_stream_mt(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStream_t st) {
     switch (pl.tnw) {
         case 4: return launch_stream<MT, 4>(a, pl, ws, st);
+        case 2: return launch_stream<MT, 2>(a, pl, ws, st);
         default: return MI355_EINVAL;
     }
 }
