@@ -1,0 +1,102 @@
+"""The entry points enqueue kernels only (no allocation, no host synchronisation, counters left zero), so a captured
+HIP graph of the quantizer + GEMM, and of the grouped GEMM, replays to the eager result every time."""
+import pytest
+import torch
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _replay_matches(fn_eager, make_graph_outputs, replays=4):
+    """fn_eager() -> tensor; make_graph_outputs() -> (graph, output tensor).  Eager work and synchronisations sit
+    between the replays, and the output is poisoned before each one."""
+    expect = fn_eager().clone()
+    graph, out = make_graph_outputs()
+    for r in range(replays):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), expect.view(torch.int16)), f"replay {r}"
+        again = fn_eager()                      # eager launches between replays share the stream's workspace
+        assert torch.equal(again.view(torch.int16), expect.view(torch.int16))
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 12288, 1024), (8, 4096, 14336), (200, 640, 8192)])
+def test_quant_and_gemm_under_graph_capture(hip, M, N, K):
+    """Persistent 256x256 launch (768 tiles), split-K stream launch, split-K 128x128 launch."""
+    from lightllm_amd.quantization import lightllm_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    print(f"graph capture gemm M={M} N={N} K={K}", flush=True)
+    x = H.activations(M, K, seed=5).cuda()
+    wq, ws = H.quantized_weights(N, K, seed=6, device="cuda")
+    xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device="cuda")
+    xs = torch.empty((M, K // 128), dtype=torch.float32, device="cuda")
+
+    def step(out):
+        lightllm_per_token_group_quant_fp8(x, 128, xq, xs)
+        w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128])
+        return out
+
+    eager_out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def capture():
+        out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(out)                            # first call on this stream allocates its workspace: before capture
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                step(out)
+        torch.cuda.current_stream().wait_stream(side)
+        return g, out
+
+    _replay_matches(lambda: step(eager_out), capture)
+
+
+def test_grouped_gemm_under_graph_capture(hip):
+    from lightllm_amd.fused_moe import grouped_matmul, moe_align_fused
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print("graph capture grouped gemm", flush=True)
+    T, E, topk, N, K = 1536, 12, 4, 2048, 1024
+    ids, tw = H.routing(T, E, topk, seed=15)
+    P = T * topk
+    idx = torch.empty((E, P), dtype=torch.int32, device="cuda")
+    w = torch.empty((E, P), dtype=torch.float32, device="cuda")
+    cnt = torch.empty((E,), dtype=torch.int32, device="cuda")
+    moe_align_fused(idx, w, cnt, ids.cuda(), tw.cuda())
+    xq, xs = per_token_group_quant_fp8(H.activations(T, K, seed=16).cuda(), 128)
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, N // 128, K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=20 + e, device="cuda")
+
+    def step(out, infos=None):
+        return grouped_matmul(P, xq, xs, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=False, use_fp8_w8a8=True,
+                              reused_mblock_infos=infos, run_config={"BLOCK_SIZE_M": 256})
+
+    eager_out = torch.empty((P, N), dtype=torch.bfloat16, device="cuda")
+    infos = step(eager_out)                     # the schedule table is built once, outside the graph
+
+    def capture():
+        out = torch.empty((P, N), dtype=torch.bfloat16, device="cuda")
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(out, infos)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                step(out, infos)
+        torch.cuda.current_stream().wait_stream(side)
+        return g, out
+
+    def eager():
+        step(eager_out, infos)
+        return eager_out
+
+    _replay_matches(eager, capture)
