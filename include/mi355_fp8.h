@@ -29,7 +29,7 @@ extern "C" {
 #define MI355_ESHAPE -2        /* shapes/strides break a precondition the reference asserts */
 #define MI355_EALIGN -3        /* a pointer or leading dimension is not aligned as the kernel needs */
 #define MI355_EWORKSPACE -4    /* workspace missing or smaller than *_workspace_bytes() */
-#define MI355_ELAUNCH -5       /* the HIP runtime refused the launch (hipGetLastError() != hipSuccess) */
+#define MI355_ELAUNCH -5       /* the HIP runtime refused the launch (hipLaunchKernel / hipFuncSetAttribute failed) */
 #define MI355_EUNSUPPORTED -6  /* valid request that no kernel variant covers */
 
 const char *mi355_error_string(int code);
@@ -45,7 +45,8 @@ int mi355_device_info(int device, int64_t out[8]);
  * replaces: lightllm_per_token_group_quant_fp8 + _per_token_group_quant_fp8
  *           (lightllm/common/basemodel/triton_kernel/quantization/fp8act_quant_kernel.py:18-113)
  *
- * x  bf16 [M,K] contiguous           (asserted there at :81)
+ * x  [M,K] contiguous (asserted there at :81); `x_dtype` MI355_DTYPE_BF16 (the hot path), _F32 or _F16:
+ *    the reference widens whatever it gets to fp32 first (:52)
  * q  e4m3fn bytes [M,K] contiguous
  * s  fp32, element (m,g) at s[m*s_stride_m + g*s_stride_g], g < K/group
  *    row-major (K/group, 1) and column-major (1, ld) are both what the reference
@@ -53,9 +54,14 @@ int mi355_device_info(int device, int64_t out[8]);
  * group must be 128 and divide K (:80); eps is the floor on the group amax (:55).
  * Arithmetic: s = max(amax,eps)/448 and q = e4m3fn_rtne(clamp(x/s,+-448)) with
  * IEEE fp32 division results, bit for bit.
+ * A group that holds a NaN or an infinity (undefined in the reference) gets s = NaN and every byte 0x7F with
+ * the sign bit of its element.
  */
-int mi355_group_quant_fp8(const void *x, void *q, float *s, int64_t M, int64_t K, int32_t group, float eps,
-                          int64_t s_stride_m, int64_t s_stride_g, void *stream);
+#define MI355_DTYPE_BF16 0
+#define MI355_DTYPE_F32 1
+#define MI355_DTYPE_F16 2
+int mi355_group_quant_fp8(const void *x, int32_t x_dtype, void *q, float *s, int64_t M, int64_t K, int32_t group,
+                          float eps, int64_t s_stride_m, int64_t s_stride_g, void *stream);
 
 /* ---------------------------------------------------------------------------
  * weight_quant (load-time 128x128 block quantizer)
@@ -64,7 +70,7 @@ int mi355_group_quant_fp8(const void *x, void *q, float *s, int64_t M, int64_t K
  *
  * w bf16 [N,K] contiguous; q e4m3fn [N,K]; s fp32 [ceil(N/128), ceil(K/128)] contiguous.
  * Keeps the reference's quirk: the stored scale is amax/448 while values are
- * divided by (scale + 1e-6), without clamp (:22-24).  `w_dtype`: 0 = bf16, 1 = fp32, 2 = fp16.
+ * divided by (scale + 1e-6), without clamp (:22-24).  `w_dtype`: MI355_DTYPE_BF16 / _F32 / _F16.
  */
 int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float *s, int64_t N, int64_t K,
                                  int32_t block, void *stream);
@@ -85,8 +91,9 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
  * C   bf16 [M,N], row stride ldc, unit column stride (:152)
  * block_n = block_k = 128.
  *
- * `variant` picks the kernel: MI355_GEMM_AUTO applies the built-in shape table; the others force
- * one (for tests and tuning).  Split-K variants need `ws` of at least
+ * `variant` picks the kernel: MI355_GEMM_AUTO applies the built-in shape table (and falls back to
+ * MI355_GEMM_TILE128 when a limit of the streaming kernel - 32-bit row offsets, workspace - is not met); the
+ * others force one (for tests and tuning) and report such a limit as an error.  Split-K variants need `ws` of at least
  * mi355_block_fp8_gemm_workspace_bytes() bytes, whose first MI355_WS_COUNTER_BYTES must be zero
  * on the first call; the kernels leave them zero again, so one zero-initialised buffer serves every call
  * issued in order on one stream.  MI355_GEMM_TILE256 uses only those counter bytes and only if it gets them:
@@ -105,7 +112,13 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
 
 #define MI355_WS_COUNTER_BYTES 65536
 
+/* Bytes of workspace the launch plan of the CURRENT device needs for this shape and variant (0 = none). */
 size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant);
+
+/* Re-zeroes the MI355_WS_COUNTER_BYTES counter bytes of a workspace (a small fill kernel on `stream`).  The
+ * kernels leave the counters zero themselves; this is the recovery path after a launch that was aborted, or
+ * after two launches were wrongly run at the same time on one workspace.  No counterpart in the reference. */
+int mi355_reset_workspace(void *ws, size_t ws_bytes, void *stream);
 
 int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C, int64_t M,
                          int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
@@ -125,6 +138,18 @@ int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const fl
 int mi355_moe_align_fused(const int32_t *topk_ids, const float *topk_weights, int64_t num_pairs,
                           int32_t num_experts, int32_t *expert_to_token_index, float *expert_to_weight,
                           int32_t *expert_token_num, void *stream);
+
+/* The two-step form of the same tables.
+ * moe_align  (grouped_fused_moe.py:39-98):   out int32 [E, num_pairs] (row stride out_stride_m), out[e, j] = 1 if
+ *            topk_ids[j] == e else 0; every element is written (the reference zero-fills first, :86).
+ * moe_align1 (grouped_fused_moe.py:101-214): compacts each row of that 0/1 table IN PLACE into the ascending pair
+ *            indices of its ones and writes the matching weights and the per-expert counts; entries past an
+ *            expert's count keep what they held. */
+int mi355_moe_align(const int32_t *topk_ids, int64_t num_pairs, int32_t num_experts, int32_t *out,
+                    int64_t out_stride_m, void *stream);
+int mi355_moe_align1(int32_t *experts_info, int64_t info_stride_m, const float *topk_weights, int64_t num_pairs,
+                     int32_t num_experts, float *experts_weight_info, int64_t weight_stride_m,
+                     int32_t *expert_token_num, void *stream);
 
 /* rows of the schedule table: min(num_pairs, ceil((num_pairs + E*(block_m-1)) / block_m))  (:457-458) */
 int64_t mi355_moe_align2_rows(int64_t num_pairs, int32_t num_experts, int32_t block_m);

@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355fp8.so")
 GEMM_AUTO, GEMM_TILE256, GEMM_TILE128, GEMM_SKINNY, GEMM_GENERIC, GEMM_TILE256x128 = 0, 1, 2, 3, 4, 5
 GEMM_TILE256_RING, GEMM_TILE256_ONCE = 6, 7
 WS_COUNTER_BYTES = 65536
+DTYPE_CODES = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}
 
 _c = ctypes
 _vp, _i64, _i32, _f32, _sz = _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_float, _c.c_size_t
@@ -19,15 +20,18 @@ _vp, _i64, _i32, _f32, _sz = _c.c_void_p, _c.c_int64, _c.c_int32, _c.c_float, _c
 SIGNATURES = {
     "mi355_error_string": (_c.c_char_p, [_c.c_int]),
     "mi355_device_info": (_c.c_int, [_c.c_int, _c.POINTER(_i64)]),
-    "mi355_group_quant_fp8": (_c.c_int, [_vp, _vp, _vp, _i64, _i64, _i32, _f32, _i64, _i64, _vp]),
+    "mi355_group_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _f32, _i64, _i64, _vp]),
     "mi355_block_weight_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp]),
     "mi355_block_fp8_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "mi355_reset_workspace": (_c.c_int, [_vp, _sz, _vp]),
     "mi355_block_fp8_gemm": (
         _c.c_int,
         [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
          _vp, _sz, _i32, _vp],
     ),
     "mi355_moe_align_fused": (_c.c_int, [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp]),
+    "mi355_moe_align": (_c.c_int, [_vp, _i64, _i32, _vp, _i64, _vp]),
+    "mi355_moe_align1": (_c.c_int, [_vp, _i64, _vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "mi355_moe_align2_rows": (_i64, [_i64, _i32, _i32]),
     "mi355_moe_align2": (_c.c_int, [_vp, _i32, _i32, _i64, _vp, _vp]),
     "mi355_grouped_block_m": (_i32, [_i64, _i32, _i64, _i64]),
@@ -95,22 +99,37 @@ def require_cuda(*tensors: torch.Tensor) -> None:
 
 
 _workspaces = {}
+_retired = []  # outgrown workspaces: kept alive, a captured HIP graph may still hold their address
 
 
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Per (device, stream) scratch for split-K and persistent launches: zero-initialised once, grown on demand.
 
-    The kernels leave the counter words zero, so the buffer is never cleared again.  Growing allocates, so
-    callers that capture HIP graphs must run each shape once before capturing (as with any torch allocator use).
+    The kernels leave the counter words zero, so the buffer is never cleared again.  A buffer that has been
+    handed out is never freed: when a later call needs more, a larger one takes its place for new launches and
+    the old one stays allocated, because a HIP graph captured earlier has its address baked in and keeps
+    using it on replay.  Growing allocates, so callers that capture graphs run each shape once before capturing
+    (as with any use of the torch allocator).
     """
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr(device))
     with _lock:
         buf = _workspaces.get(key)
         if buf is None or buf.numel() < nbytes:
+            if buf is not None:
+                _retired.append(buf)
             size = max(nbytes, WS_COUNTER_BYTES + (32 << 20))
             buf = torch.zeros(size, dtype=torch.uint8, device=device)
             _workspaces[key] = buf
     return buf
+
+
+def reset_workspace(device: torch.device) -> None:
+    """Re-zero the counter words of the current stream's workspace (after an aborted launch)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr(device))
+    with _lock:
+        buf = _workspaces.get(key)
+    if buf is not None:
+        check(lib().mi355_reset_workspace(buf.data_ptr(), buf.numel(), stream_ptr(device)), "mi355_reset_workspace")
 
 
 def device_info(device: int = -1) -> dict:

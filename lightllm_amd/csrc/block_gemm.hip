@@ -1,6 +1,5 @@
 // Host side of the block-scaled FP8 GEMM entry points: argument checks, kernel choice, launches.
 #include <cstdlib>
-#include <mutex>
 
 #include "gemm_pp.hpp"
 #include "gemm_stream.hpp"
@@ -39,12 +38,6 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_generic_kernel(
 
 constexpr int kMaxLds = 160 * 1024;  // LDS per workgroup on gfx950
 
-template <typename KernelT>
-static hipError_t allow_lds(KernelT kernel, int bytes) {
-    // Raising the dynamic-LDS ceiling is a per-function host-side setting; it enqueues nothing.
-    return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 // X scales that can be fetched eight K steps at a time: row-major, 16-byte aligned rows, K/128 % 8 == 0.
 static bool chunked_scales_ok(const GemmArgs &a) {
     return a.xs_k == 1 && (a.K / kBlockK) % 8 == 0 && a.xs_m % 4 == 0 && ((uintptr_t)a.Xs & 15) == 0;
@@ -53,17 +46,13 @@ static bool chunked_scales_ok(const GemmArgs &a) {
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
 static int launch_tile_as(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
-    auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE, XS8>;
+    constexpr auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE, XS8>;
     const int KB = a.K / kBlockK;
     // chunked scales keep two [BM rows][8 steps] buffers behind the common layout
     const int lds_bytes = XS8 ? ((Cfg::lds_bytes(KB) + 127) & ~127) + 2 * BM * 32 : Cfg::lds_bytes(KB);
     if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] { attr_err = allow_lds(kernel, kMaxLds); });
-    if (attr_err != hipSuccess) return MI355_ELAUNCH;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::kThreads), lds_bytes, st, a);
-    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+    if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
+    return launch(kernel, dim3(grid), dim3(Cfg::kThreads), lds_bytes, st, a);
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
@@ -88,11 +77,8 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hipStream_
     if (!chunked_scales_ok(a)) return MI355_EUNSUPPORTED;
     const int lds_bytes = PPCfg::lds_bytes(a.K / kBlockK);
     if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
-    auto kernel = block_fp8_gemm_pp_kernel<GROUPED>;
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] { attr_err = allow_lds(kernel, kMaxLds); });
-    if (attr_err != hipSuccess) return MI355_ELAUNCH;
+    constexpr auto kernel = block_fp8_gemm_pp_kernel<GROUPED>;
+    if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
     a.blocks_per_xcd = (a.total_tiles + 7) / 8;
     int per_xcd = a.blocks_per_xcd;
     a.counters = nullptr;
@@ -101,8 +87,7 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hipStream_
         a.counters = (uint32_t *)ws;
         per_xcd = cus / 8;
     }
-    hipLaunchKernelGGL(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_bytes, st, a);
-    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+    return launch(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_bytes, st, a);
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE = kDense>
@@ -141,28 +126,33 @@ static size_t skinny_workspace(int64_t M, const SkinnyPlan &pl) {
     return (size_t)MI355_WS_COUNTER_BYTES + (size_t)pl.tiles * pl.splits * 16 * skinny_mt(M) * 16 * pl.tnw * 4;
 }
 
+// Preconditions of the stream kernel beyond the fast layout.
+static int skinny_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t as_m, int cus,
+                        const void *ws, size_t ws_bytes) {
+    if (M > 64) return MI355_EUNSUPPORTED;
+    // rows are addressed from the matrix bases with 32-bit byte offsets
+    if (N * ldw >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)) return MI355_EUNSUPPORTED;
+    const SkinnyPlan pl = skinny_plan(M, N, K, cus);
+    if ((int64_t)pl.tiles * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
+    if (pl.splits > 1 && (!ws || ws_bytes < skinny_workspace(M, pl) || ((uintptr_t)ws & 15))) return MI355_EWORKSPACE;
+    return MI355_OK;
+}
+
 template <int MT, int TNW, bool XSL>
 static int launch_stream_as(GemmArgs &a, const SkinnyPlan &pl, void *ws, int lds_bytes, hipStream_t st) {
     using Cfg = StreamCfg<MT, TNW>;
-    static std::once_flag once;
-    static hipError_t e0 = hipSuccess, e1 = hipSuccess;
-    std::call_once(once, [&] {
-        const int max_lds = Cfg::kLds + (XSL ? Cfg::scale_lds_bytes(Cfg::kMaxScaleSteps) : 0);
-        e0 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, false, XSL>, max_lds);
-        e1 = allow_lds(block_fp8_gemm_stream_kernel<MT, TNW, true, XSL>, max_lds);
-    });
-    if (e0 != hipSuccess || e1 != hipSuccess) return MI355_ELAUNCH;
+    constexpr int max_lds = Cfg::kLds + (XSL ? Cfg::scale_lds_bytes(Cfg::kMaxScaleSteps) : 0);
+    constexpr auto whole_k = block_fp8_gemm_stream_kernel<MT, TNW, false, XSL>;
+    constexpr auto split_k = block_fp8_gemm_stream_kernel<MT, TNW, true, XSL>;
     if (pl.splits <= 1) {
-        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, false, XSL>), dim3(pl.tiles), dim3(256), lds_bytes, st,
-                           a);
-    } else {
-        a.splits = pl.splits;
-        a.counters = (uint32_t *)ws;
-        a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
-        hipLaunchKernelGGL((block_fp8_gemm_stream_kernel<MT, TNW, true, XSL>), dim3(pl.tiles * pl.splits), dim3(256),
-                           lds_bytes, st, a);
+        if (!allow_lds<whole_k>(max_lds)) return MI355_ELAUNCH;
+        return launch(whole_k, dim3(pl.tiles), dim3(256), lds_bytes, st, a);
     }
-    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+    if (!allow_lds<split_k>(max_lds)) return MI355_ELAUNCH;
+    a.splits = pl.splits;
+    a.counters = (uint32_t *)ws;
+    a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+    return launch(split_k, dim3(pl.tiles * pl.splits), dim3(256), lds_bytes, st, a);
 }
 
 // The activation scales of a CTA's K range are staged in LDS when the range is short enough for the staging area.
@@ -183,18 +173,6 @@ static int launch_stream_mt(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStre
         case 2: return launch_stream<MT, 2>(a, pl, ws, st);
         default: return MI355_EINVAL;
     }
-}
-
-static int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
-    return cus;
 }
 
 static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n) {
@@ -232,16 +210,18 @@ using namespace mi355;
 
 extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, 256);
     if (K % kBlockK != 0) return 0;
+    // sized from the launch plan of the current device (256 compute units when no device is visible)
+    const int cus = device_cus();
+    if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, cus);
     if (variant == MI355_GEMM_TILE128) {
-        const int splits = tile128_splits(M, N, K, 256);
-        return splits > 1 ? tile128_workspace(M, N, splits) * 2 : 0;  // x2: headroom for devices with more CUs
+        const int splits = tile128_splits(M, N, K, cus);
+        return splits > 1 ? tile128_workspace(M, N, splits) : 0;
     }
     if (variant == MI355_GEMM_TILE256) return MI355_WS_COUNTER_BYTES;  // the tile counters of the persistent launch
     if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
-    // sized for the deepest split (a one-CU device), so the figure does not depend on the device
-    return skinny_workspace(M, skinny_plan(M, N, K, 1 << 20));
+    const SkinnyPlan pl = skinny_plan(M, N, K, cus);
+    return pl.splits > 1 ? skinny_workspace(M, pl) : 0;
 }
 
 extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C,
@@ -263,16 +243,21 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
                       // 32-bit byte offsets inside a tile / scale column
                       256 * lda < (1ll << 32) && 256 * ldb_n < (1ll << 32) && 256 * as_m * 4 < (1ll << 32) &&
                       as_m >= 0 && as_k >= 0;
-    if (variant == MI355_GEMM_AUTO) variant = fast ? pick_variant(M, N, cus) : MI355_GEMM_GENERIC;
+    if (variant == MI355_GEMM_AUTO) {
+        variant = fast ? pick_variant(M, N, cus) : MI355_GEMM_GENERIC;
+        // the stream kernel's own limits are not errors under AUTO: the 128x128 tile takes every fast layout
+        // and runs unsplit without a workspace
+        if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
+            variant = MI355_GEMM_TILE128;
+    }
     if (variant != MI355_GEMM_GENERIC && !fast) return MI355_EALIGN;
 
     if (variant == MI355_GEMM_GENERIC) {
         const int64_t blocks = (M * N + 255) / 256;
         if (blocks >= (1ll << 31)) return MI355_EUNSUPPORTED;
-        hipLaunchKernelGGL(block_fp8_gemm_generic_kernel, dim3((uint32_t)blocks), dim3(256), 0, st,
-                           (const uint8_t *)A, (const uint8_t *)B, As, Bs, (uint16_t *)C, (int)M, (int)N, (int)K, lda,
-                           ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n, (int)block_n, (int)block_k);
-        return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
+        return launch(block_fp8_gemm_generic_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, (const uint8_t *)A,
+                      (const uint8_t *)B, As, Bs, (uint16_t *)C, (int)M, (int)N, (int)K, lda, ldb_k, ldb_n, ldc, as_m,
+                      as_k, bs_k, bs_n, (int)block_n, (int)block_k);
     }
 
     GemmArgs a = {};
@@ -324,13 +309,9 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
             return launch_tile<128, 128, 2, 2, 2, kSplitK>(a, a.total_tiles * splits, st);
         }
         case MI355_GEMM_SKINNY: {
-            if (M > 64) return MI355_EUNSUPPORTED;
-            // the stream kernel addresses rows from the matrix bases with 32-bit byte offsets
-            if (N * ldb_n >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)) return MI355_EUNSUPPORTED;
+            const int ok = skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes);
+            if (ok != MI355_OK) return ok;
             const SkinnyPlan pl = skinny_plan(M, N, K, cus);
-            if ((int64_t)pl.tiles * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
-            if (pl.splits > 1 && (!ws || ws_bytes < skinny_workspace(M, pl) || ((uintptr_t)ws & 15)))
-                return MI355_EWORKSPACE;
             switch (skinny_mt(M)) {
                 case 1: return launch_stream_mt<1>(a, pl, ws, st);
                 case 2: return launch_stream_mt<2>(a, pl, ws, st);
@@ -340,6 +321,22 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
         default:
             return MI355_EINVAL;
     }
+}
+
+namespace mi355 {
+
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+}  // namespace mi355
+
+/* Re-zeroes the counter words of a caller-owned workspace (recovery after an aborted launch). */
+extern "C" int mi355_reset_workspace(void *ws, size_t ws_bytes, void *stream) {
+    if (!ws || ws_bytes < (size_t)MI355_WS_COUNTER_BYTES || ((uintptr_t)ws & 3)) return MI355_EWORKSPACE;
+    const uint32_t words = MI355_WS_COUNTER_BYTES / 4;
+    return launch(zero_words_kernel, dim3(words / 256), dim3(256), 0, (hipStream_t)stream, (uint32_t *)ws, words);
 }
 
 extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K) {

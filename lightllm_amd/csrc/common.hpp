@@ -3,6 +3,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <tuple>
+#include <utility>
+
 #include "../../include/mi355_fp8.h"
 
 namespace mi355 {
@@ -81,5 +85,62 @@ __device__ __forceinline__ void wait_vmcnt() {
 // distinct, and for 8 consecutive rows the physical chunks are all distinct, so a ds_read_b128 of a
 // 16-row operand slice is bank-conflict free whether the LDS serves 128 or 256 bytes per clock.
 __device__ __forceinline__ uint32_t swz(uint32_t row) { return (row & 7u) ^ ((row >> 3) & 1u); }
+
+// ---- host side: launches and per-device facts ------------------------------------------------------------
+// A launch reports the status of its own hipLaunchKernel call.  (hipGetLastError() after a <<<>>> launch
+// would also return, and clear, an error left behind by an unrelated earlier runtime call of the host
+// framework.)
+namespace detail {
+template <typename... P, size_t... I>
+inline hipError_t launch_impl(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t st,
+                              std::tuple<P...> &params, std::index_sequence<I...>) {
+    void *ptrs[] = {(void *)&std::get<I>(params)...};
+    return hipLaunchKernel((const void *)kernel, grid, block, ptrs, lds, st);
+}
+}  // namespace detail
+
+template <typename... P, typename... A>
+inline int launch(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds, hipStream_t st, A &&...args) {
+    static_assert(sizeof...(P) == sizeof...(A), "argument count differs from the kernel's parameter list");
+    std::tuple<P...> params{static_cast<P>(args)...};
+    return detail::launch_impl(kernel, grid, block, lds, st, params, std::index_sequence_for<P...>{}) == hipSuccess
+               ? MI355_OK
+               : MI355_ELAUNCH;
+}
+
+constexpr int kMaxDevices = 64;
+
+inline int current_device() {
+    int dev = 0;
+    return hipGetDevice(&dev) == hipSuccess ? dev : -1;
+}
+
+// Compute units of the current device (looked up once per device).
+inline int device_cus() {
+    static std::atomic<int> cus[kMaxDevices];
+    const int dev = current_device();
+    if (dev >= 0 && dev < kMaxDevices) {
+        const int known = cus[dev].load(std::memory_order_relaxed);
+        if (known > 0) return known;
+    }
+    int n = 0;
+    if (dev < 0 || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    if (dev >= 0 && dev < kMaxDevices) cus[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+// Raises the dynamic-LDS ceiling of Kernel to `bytes` on the current device, once per device: the attribute
+// belongs to the device's copy of the function.  Setting it enqueues nothing.
+template <auto Kernel>
+inline bool allow_lds(int bytes) {
+    static std::atomic<uint64_t> done{0};
+    const int dev = current_device();
+    const bool tracked = dev >= 0 && dev < kMaxDevices;
+    if (tracked && ((done.load(std::memory_order_acquire) >> dev) & 1u)) return true;
+    if (hipFuncSetAttribute((const void *)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+        return false;
+    if (tracked) done.fetch_or(1ull << dev, std::memory_order_release);
+    return true;
+}
 
 }  // namespace mi355

@@ -1,6 +1,6 @@
 // per_token_group_quant_fp8 for gfx950: an HBM-streaming kernel.
 //
-// Data layout: x is bf16 [M,K] contiguous, so every group of 128 elements is 256 contiguous bytes
+// Data layout (bf16, the hot path): x is [M,K] contiguous, so every group of 128 elements is 256 contiguous bytes
 // and the whole tensor is a flat array of 16-byte chunks (8 bf16).  One lane owns one chunk; the 16
 // lanes of a DPP row own one group; a wave covers 4 groups (1 KiB) per load instruction and keeps
 // UNROLL such loads in flight.  The group amax is reduced inside the DPP row (4 steps), the scale
@@ -48,13 +48,48 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const v4i *__restrict_
     }
 }
 
+// fp16 and fp32 activations (the reference widens any input dtype to fp32 first,
+// quantization/fp8act_quant_kernel.py:52): one lane = 8 elements, true divisions.  Not the hot path.
+template <typename T>
+__global__ __launch_bounds__(256) void group_quant_wide_kernel(const T *__restrict__ x, v2i *__restrict__ q,
+                                                               float *__restrict__ s, uint32_t total_chunks,
+                                                               uint32_t groups_per_row, int64_t s_stride_m,
+                                                               int64_t s_stride_g, float eps) {
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c >= total_chunks) return;  // total_chunks is a multiple of 16: a DPP row is active or idle as a whole
+    float f[8];
+    if constexpr (sizeof(T) == 4) {
+        const v4i a = __builtin_nontemporal_load((const v4i *)x + 2 * (size_t)c);
+        const v4i b = __builtin_nontemporal_load((const v4i *)x + 2 * (size_t)c + 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[i] = as_f32((uint32_t)a[i]);
+            f[4 + i] = as_f32((uint32_t)b[i]);
+        }
+    } else {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        const h8 h = __builtin_bit_cast(h8, __builtin_nontemporal_load((const v4i *)x + c));
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)h[i];
+    }
+    v2i o;
+    float sc;
+    quant_chunk_f32(f, eps, o, sc);
+    __builtin_nontemporal_store(o, q + c);
+    if ((threadIdx.x & 15u) == 0) {
+        const uint32_t g = c >> 4;
+        const uint32_t row = g / groups_per_row, col = g - row * groups_per_row;
+        s[(int64_t)row * s_stride_m + (int64_t)col * s_stride_g] = sc;
+    }
+}
+
 }  // namespace mi355
 
 using namespace mi355;
 
-extern "C" int mi355_group_quant_fp8(const void *x, void *q, float *s, int64_t M, int64_t K, int32_t group,
-                                     float eps, int64_t s_stride_m, int64_t s_stride_g, void *stream) {
-    if (M < 0 || K < 0) return MI355_EINVAL;
+extern "C" int mi355_group_quant_fp8(const void *x, int32_t x_dtype, void *q, float *s, int64_t M, int64_t K,
+                                     int32_t group, float eps, int64_t s_stride_m, int64_t s_stride_g, void *stream) {
+    if (M < 0 || K < 0 || x_dtype < 0 || x_dtype > 2) return MI355_EINVAL;
     if (group != 128) return MI355_EUNSUPPORTED;
     if (K % group != 0) return MI355_ESHAPE;
     if (M == 0 || K == 0) return MI355_OK;
@@ -69,11 +104,16 @@ extern "C" int mi355_group_quant_fp8(const void *x, void *q, float *s, int64_t M
     constexpr int UNROLL = 4;
     uint32_t blocks = (uint32_t)((chunks + 256 * UNROLL - 1) / (256 * UNROLL));
     hipStream_t st = (hipStream_t)stream;
+    if (x_dtype == MI355_DTYPE_F32)
+        return launch(group_quant_wide_kernel<float>, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
+                      (const float *)x, (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps);
+    if (x_dtype == MI355_DTYPE_F16)
+        return launch(group_quant_wide_kernel<_Float16>, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
+                      (const _Float16 *)x, (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps);
     if (row_major)
-        hipLaunchKernelGGL((group_quant_kernel<UNROLL, true>), dim3(blocks), dim3(256), 0, st, (const v4i *)x,
+        return launch((group_quant_kernel<UNROLL, true>), dim3(blocks), dim3(256), 0, st, (const v4i *)x,
                            (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps, eps_default);
     else
-        hipLaunchKernelGGL((group_quant_kernel<UNROLL, false>), dim3(blocks), dim3(256), 0, st, (const v4i *)x,
+        return launch((group_quant_kernel<UNROLL, false>), dim3(blocks), dim3(256), 0, st, (const v4i *)x,
                            (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps, eps_default);
-    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
 }

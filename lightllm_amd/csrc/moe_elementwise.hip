@@ -251,8 +251,6 @@ __global__ __launch_bounds__(256) void weight_dequant_scalar_kernel(const uint8_
     out[i] = (uint16_t)f32_to_bf16_bits_nan(a[0] * s[(row >> 7) * kblocks + (col >> 7)]);
 }
 
-static inline bool launched() { return hipGetLastError() == hipSuccess; }
-
 }  // namespace mi355
 
 using namespace mi355;
@@ -272,15 +270,14 @@ extern "C" int mi355_silu_and_mul(const void *in, void *out, int64_t M, int64_t 
         constexpr int UNROLL = 4;
         const uint32_t cpr = (uint32_t)(H / 8);
         uint32_t blocks = (uint32_t)((chunks + 256 * UNROLL - 1) / (256 * UNROLL));
-        hipLaunchKernelGGL((silu_and_mul_kernel<UNROLL>), dim3(blocks), dim3(256), 0, st, (const uint16_t *)in,
+        return launch((silu_and_mul_kernel<UNROLL>), dim3(blocks), dim3(256), 0, st, (const uint16_t *)in,
                            (uint16_t *)out, (uint32_t)chunks, cpr, 256u / cpr, 256u % cpr, in_stride_m, out_stride_m);
     } else {
         int64_t total = M * H;
         if ((total + 255) / 256 >= (int64_t)1 << 31) return MI355_EUNSUPPORTED;
-        hipLaunchKernelGGL(silu_and_mul_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
+        return launch(silu_and_mul_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
                            (const uint16_t *)in, (uint16_t *)out, total, H, in_stride_m, out_stride_m);
     }
-    return launched() ? MI355_OK : MI355_ELAUNCH;
 }
 
 extern "C" int mi355_silu_and_mul_group_quant_fp8(const void *in, void *q, float *s, int64_t M, int64_t H,
@@ -302,14 +299,13 @@ extern "C" int mi355_silu_and_mul_group_quant_fp8(const void *in, void *q, float
     uint32_t blocks = (uint32_t)((chunks + 256 * UNROLL - 1) / (256 * UNROLL));
     hipStream_t st = (hipStream_t)stream;
     if (masked_m)
-        hipLaunchKernelGGL((silu_mul_quant_kernel<UNROLL, true>), dim3(blocks), dim3(256), 0, st,
+        return launch((silu_mul_quant_kernel<UNROLL, true>), dim3(blocks), dim3(256), 0, st,
                            (const uint16_t *)in, (v2i *)q, s, (uint32_t)chunks, cpr, 256u / cpr, 256u % cpr,
                            in_stride_m, s_stride_m, s_stride_g, masked_m, (uint32_t)rows_per_expert);
     else
-        hipLaunchKernelGGL((silu_mul_quant_kernel<UNROLL, false>), dim3(blocks), dim3(256), 0, st,
+        return launch((silu_mul_quant_kernel<UNROLL, false>), dim3(blocks), dim3(256), 0, st,
                            (const uint16_t *)in, (v2i *)q, s, (uint32_t)chunks, cpr, 256u / cpr, 256u % cpr,
                            in_stride_m, s_stride_m, s_stride_g, masked_m, 1u);
-    return launched() ? MI355_OK : MI355_ELAUNCH;
 }
 
 extern "C" int mi355_moe_sum_reduce(const void *in, void *out, int64_t T, int32_t topk, int64_t H, void *stream) {
@@ -320,15 +316,14 @@ extern "C" int mi355_moe_sum_reduce(const void *in, void *out, int64_t T, int32_
     if (H % 8 == 0 && !((uintptr_t)in & 15) && !((uintptr_t)out & 15)) {
         int64_t chunks = T * (H / 8);
         if (chunks >= (int64_t)1 << 32) return MI355_EUNSUPPORTED;
-        hipLaunchKernelGGL((moe_sum_reduce_kernel<4>), dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
+        return launch((moe_sum_reduce_kernel<4>), dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
                            (const v4i *)in, (v4i *)out, (uint32_t)chunks, (uint32_t)(H / 8), topk);
     } else {
         int64_t total = T * H;
         if ((total + 255) / 256 >= (int64_t)1 << 31) return MI355_EUNSUPPORTED;
-        hipLaunchKernelGGL(moe_sum_reduce_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
+        return launch(moe_sum_reduce_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
                            (const uint16_t *)in, (uint16_t *)out, total, H, topk);
     }
-    return launched() ? MI355_OK : MI355_ELAUNCH;
 }
 
 extern "C" int mi355_block_weight_dequant(const void *q, const float *s, void *out, int64_t N, int64_t K,
@@ -342,13 +337,12 @@ extern "C" int mi355_block_weight_dequant(const void *q, const float *s, void *o
     if (K % 16 == 0 && !((uintptr_t)q & 15) && !((uintptr_t)out & 15)) {
         int64_t chunks = N * (K / 16);
         if (chunks >= (int64_t)1 << 32) return MI355_EUNSUPPORTED;
-        hipLaunchKernelGGL(weight_dequant_kernel, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
+        return launch(weight_dequant_kernel, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
                            (const v4i *)q, s, (v4i *)out, (uint32_t)chunks, (uint32_t)(K / 16), (uint32_t)kblocks);
     } else {
         int64_t total = N * K;
         if ((total + 255) / 256 >= (int64_t)1 << 31) return MI355_EUNSUPPORTED;
-        hipLaunchKernelGGL(weight_dequant_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
+        return launch(weight_dequant_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
                            (const uint8_t *)q, s, (uint16_t *)out, total, K, kblocks);
     }
-    return launched() ? MI355_OK : MI355_ELAUNCH;
 }

@@ -1,4 +1,4 @@
-// Device-side arithmetic of the 1x128 group quantizer (bf16 -> e4m3fn + fp32 scale), shared by the
+// Device-side arithmetic of the 1x128 group quantizer (bf16 / fp16 / fp32 -> e4m3fn + fp32 scale), shared by the
 // stand-alone quantizer and by the kernels that quantize what they have just computed.
 //
 // Arithmetic (must reproduce IEEE fp32 division results bit for bit, see
@@ -50,7 +50,51 @@ __device__ __forceinline__ float quot(float x, float s, float r) {
     return as_f32((as_u32(y) & 0x7fffffffu) | (as_u32(x) & 0x80000000u));
 }
 
-// Quantize one 16-byte chunk; the group amax is shared through the DPP row.
+// A group that holds a NaN or an infinity (outside the reference's contract: its max and clamp leave NaN
+// unspecified) is poisoned as a whole: scale = NaN, every byte 0x7F with the sign bit of its element.
+__device__ __forceinline__ void nonfinite_chunk(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t s3, uint32_t s4,
+                                                uint32_t s5, uint32_t s6, uint32_t s7, v2i &out, float &scale) {
+    out[0] = (int)(0x7f7f7f7fu | (s0 << 7) | (s1 << 15) | (s2 << 23) | (s3 << 31));
+    out[1] = (int)(0x7f7f7f7fu | (s4 << 7) | (s5 << 15) | (s6 << 23) | (s7 << 31));
+    scale = as_f32(0x7fc00000u);
+}
+
+// Quantize 8 consecutive fp32 values (fp16 / fp32 activations, widened by the caller) with true IEEE divisions:
+// the two-FMA quotient above is only proven for bf16 inputs.
+__device__ __forceinline__ void quant_chunk_f32(const float (&f)[8], float eps, v2i &out, float &scale) {
+    uint32_t mx = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t a = as_u32(f[i]) & 0x7fffffffu;
+        mx = a > mx ? a : mx;
+    }
+    mx = row16_max_u32(mx);
+    if (mx > 0x7f7fffffu) {
+        nonfinite_chunk(as_u32(f[0]) >> 31, as_u32(f[1]) >> 31, as_u32(f[2]) >> 31, as_u32(f[3]) >> 31,
+                        as_u32(f[4]) >> 31, as_u32(f[5]) >> 31, as_u32(f[6]) >> 31, as_u32(f[7]) >> 31, out, scale);
+        return;
+    }
+    float amax = as_f32(mx);
+    amax = amax > eps ? amax : eps;
+    const float s = amax / 448.0f;
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        y[i] = f[i] / s;
+        y[i] = y[i] > 448.0f ? 448.0f : y[i];
+        y[i] = y[i] < -448.0f ? -448.0f : y[i];
+    }
+    int w0 = 0, w1 = 0;
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], w0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], w1, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+    out[0] = w0;
+    out[1] = w1;
+    scale = s;
+}
+
+// Quantize one 16-byte chunk of bf16; the group amax is shared through the DPP row.
 __device__ __forceinline__ void quant_chunk(const v4i &v, float eps, bool eps_is_default, v2i &out, float &scale) {
     uint32_t d0 = (uint32_t)v[0], d1 = (uint32_t)v[1], d2 = (uint32_t)v[2], d3 = (uint32_t)v[3];
     // |x| as integers: for non-negative floats the integer order is the float order.
@@ -59,6 +103,11 @@ __device__ __forceinline__ void quant_chunk(const v4i &v, float eps, bool eps_is
     uint32_t hi = m >> 16, lo = m & 0xffffu;
     uint32_t mx = (hi > lo ? hi : lo) << 16;
     mx = row16_max_u32(mx);
+    if (mx > 0x7f7fffffu) {  // the same for all 16 lanes of the group
+        nonfinite_chunk((d0 >> 15) & 1u, d0 >> 31, (d1 >> 15) & 1u, d1 >> 31, (d2 >> 15) & 1u, d2 >> 31,
+                        (d3 >> 15) & 1u, d3 >> 31, out, scale);
+        return;
+    }
     float amax = as_f32(mx);
     amax = amax > eps ? amax : eps;
     float s;

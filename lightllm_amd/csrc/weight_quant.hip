@@ -125,16 +125,15 @@ extern "C" int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void
     dim3 grid((uint32_t)kb, (uint32_t)nb);
     hipStream_t st = (hipStream_t)stream;
     if (w_dtype == 0 && K % 8 == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)q & 7) == 0)
-        hipLaunchKernelGGL(block_weight_quant_bf16_kernel, grid, dim3(256), 0, st, (const uint16_t *)w, (uint8_t *)q, s,
+        return launch(block_weight_quant_bf16_kernel, grid, dim3(256), 0, st, (const uint16_t *)w, (uint8_t *)q, s,
                            N, K, (int)kb);
     else if (w_dtype == 0)
-        hipLaunchKernelGGL(block_weight_quant_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t *)w,
+        return launch(block_weight_quant_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t *)w,
                            (uint8_t *)q, s, N, K, (int)kb);
     else if (w_dtype == 1)
-        hipLaunchKernelGGL(block_weight_quant_kernel<float>, grid, dim3(256), 0, st, (const float *)w, (uint8_t *)q, s,
+        return launch(block_weight_quant_kernel<float>, grid, dim3(256), 0, st, (const float *)w, (uint8_t *)q, s,
                            N, K, (int)kb);
     else
-        hipLaunchKernelGGL(block_weight_quant_kernel<_Float16>, grid, dim3(256), 0, st, (const _Float16 *)w,
+        return launch(block_weight_quant_kernel<_Float16>, grid, dim3(256), 0, st, (const _Float16 *)w,
                            (uint8_t *)q, s, N, K, (int)kb);
-    return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ELAUNCH;
 }

@@ -1,4 +1,11 @@
-from .grouped_fused_moe import fused_experts_impl, grouped_matmul, moe_align2, moe_align_fused  # noqa: F401
+from .grouped_fused_moe import (  # noqa: F401
+    fused_experts_impl,
+    grouped_matmul,
+    moe_align,
+    moe_align1,
+    moe_align2,
+    moe_align_fused,
+)
 from .moe_silu_and_mul import silu_and_mul_fwd  # noqa: F401
 from .moe_silu_and_mul_mix_quant_ep import (  # noqa: F401
     silu_and_mul_masked_post_quant_fwd,

@@ -2,7 +2,7 @@
 
 Same names, arguments and tensor layouts as
 lightllm/common/basemodel/triton_kernel/fused_moe/grouped_fused_moe.py of the reference
-(moe_align_fused :388-396, moe_align2 :452-477, grouped_matmul :771-989, fused_experts_impl :992-1115);
+(moe_align :64-98, moe_align1 :147-214, moe_align_fused :388-396, moe_align2 :452-477, grouped_matmul :771-989, fused_experts_impl :992-1115);
 the work is done by ``mi355_moe_align_fused``, ``mi355_moe_align2`` and ``mi355_grouped_block_fp8_gemm``.
 Only the fp8 128x128-block branch exists here (use_fp8_w8a8=True with 3-D weight scales).
 """
@@ -17,6 +17,44 @@ from .moe_sum_reduce import moe_sum_reduce
 
 _BLOCK_MS = (16, 32, 64, 128, 256)
 FFN_MOE_CHUNK_SIZE = 32 * 1024  # tokens per pass of fused_experts_impl (reference :34)
+
+
+def moe_align(topk_ids: torch.Tensor, out: torch.Tensor):
+    """out int32 [E, T*topk]: out[e, j] = 1 where the flattened pair j of ``topk_ids`` [T, topk] is routed to
+    expert e, 0 elsewhere (reference :64-98; its zero fill is part of the kernel here)."""
+    token_num, topk = topk_ids.shape
+    assert out.shape[1] == token_num * topk, f"out shape {out.shape} topk_ids shape {topk_ids.shape} "
+    assert topk_ids.is_contiguous()
+    assert topk_ids.dtype == torch.int32 and out.dtype == torch.int32 and out.stride(1) == 1
+    _lib.require_cuda(topk_ids, out)
+    code = _lib.lib().mi355_moe_align(
+        topk_ids.data_ptr(), token_num * topk, out.shape[0], out.data_ptr(), out.stride(0),
+        _lib.stream_ptr(out.device),
+    )
+    _lib.check(code, "moe_align")
+
+
+def moe_align1(experts_info: torch.Tensor, topk_weights: torch.Tensor, experts_weight_info: torch.Tensor,
+               exports_token_num: torch.Tensor, topk: int):
+    """Compacts the 0/1 table of ``moe_align`` in place into pair indices, with the weights and the per-expert
+    counts (reference :147-214).  Entries past an expert's count keep what they held."""
+    expert_num, token_num_mul_topk = experts_info.shape
+    topk_num = topk_weights.shape[1]
+    assert token_num_mul_topk <= FFN_MOE_CHUNK_SIZE * topk_num, "need split to handle seq len too long"
+    assert exports_token_num.shape[0] == expert_num
+    assert topk_weights.is_contiguous()
+    assert experts_info.dtype == torch.int32 and experts_info.stride(1) == 1
+    assert experts_weight_info.dtype == torch.float32 and experts_weight_info.stride(1) == 1
+    assert experts_weight_info.shape == experts_info.shape
+    assert exports_token_num.dtype == torch.int32 and exports_token_num.is_contiguous()
+    assert topk_weights.dtype == torch.float32
+    _lib.require_cuda(experts_info, topk_weights, experts_weight_info, exports_token_num)
+    code = _lib.lib().mi355_moe_align1(
+        experts_info.data_ptr(), experts_info.stride(0), topk_weights.data_ptr(), token_num_mul_topk, expert_num,
+        experts_weight_info.data_ptr(), experts_weight_info.stride(0), exports_token_num.data_ptr(),
+        _lib.stream_ptr(experts_info.device),
+    )
+    _lib.check(code, "moe_align1")
 
 
 def moe_align_fused(expert_to_token_index, expert_to_weight, expert_token_num, topk_ids, topk_weights):

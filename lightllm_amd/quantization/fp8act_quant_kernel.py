@@ -1,4 +1,4 @@
-"""Activation quantizer: bf16 -> float8_e4m3fn with one fp32 scale per 1x128 group.
+"""Activation quantizer: bf16 (fp16, fp32) -> float8_e4m3fn with one fp32 scale per 1x128 group.
 
 Same names, arguments and tensor layouts as
 lightllm/common/basemodel/triton_kernel/quantization/fp8act_quant_kernel.py (:63-113, :116-168, :216-236)
@@ -33,7 +33,7 @@ def lightllm_per_token_group_quant_fp8(
     assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
     assert x.is_contiguous(), "`x` is not contiguous"
     assert dtype == torch.float8_e4m3fn, "only torch.float8_e4m3fn is supported"
-    assert x.dtype == torch.bfloat16, "the gfx950 quantizer takes bf16 activations"
+    assert x.dtype in _lib.DTYPE_CODES, "activations must be bf16 (the fast path), fp16 or fp32"
     assert x_q.is_contiguous() and x_q.shape == x.shape and x_q.dtype == torch.float8_e4m3fn
     assert x_s.dtype == torch.float32
     _lib.require_cuda(x, x_q, x_s)
@@ -42,7 +42,8 @@ def lightllm_per_token_group_quant_fp8(
     M = x.numel() // K if K else 0
     assert xs_m == M and xs_n == K // group_size, "scale tensor shape must be [M, K // group_size]"
     code = _lib.lib().mi355_group_quant_fp8(
-        x.data_ptr(), x_q.data_ptr(), x_s.data_ptr(), M, K, group_size, eps, x_s.stride(0), x_s.stride(1),
+        x.data_ptr(), _lib.DTYPE_CODES[x.dtype], x_q.data_ptr(), x_s.data_ptr(), M, K, group_size, eps,
+        x_s.stride(0), x_s.stride(1),
         _lib.stream_ptr(x.device),
     )
     _lib.check(code, "per_token_group_quant_fp8")

@@ -35,8 +35,7 @@ def build(force: bool = False) -> str:
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
-            build()
+        build()  # no-op unless the library is missing or older than its source
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.oracle_moe_align2_rows.restype = ctypes.c_int64
         _lib.oracle_moe_align2_rows.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
@@ -105,6 +104,18 @@ def group_quant_fp8(x_bf16_bits, group: int = 128, eps: float = 1e-10, column_ma
     return q, s
 
 
+def group_quant_fp8_f32(x_f32, group: int = 128, eps: float = 1e-10):
+    """x: float32 [M,K] (fp16 and bf16 inputs widen exactly) -> (q uint8 [M,K], s float32 [M,K/group])."""
+    x = _c(x_f32, np.float32)
+    M, K = x.shape
+    assert K % group == 0
+    G = K // group
+    q = np.empty((M, K), np.uint8)
+    s = np.empty((M, G), np.float32)
+    lib().oracle_group_quant_fp8_f32(_p(x), I64(M), I64(K), I32(group), F32(eps), _p(q), _p(s), I64(G), I64(1))
+    return q, s
+
+
 def block_weight_quant(w_f32, block: int = 128):
     """w: float32 [N,K] -> (q uint8 [N,K], s float32 [ceil(N/b), ceil(K/b)])."""
     w = _c(w_f32, np.float32)
@@ -152,6 +163,25 @@ def moe_align_fused(topk_ids, topk_weights, num_experts: int):
     cnt = np.empty((num_experts,), np.int32)
     lib().oracle_moe_align_fused(_p(ids), _p(w), I64(P), I32(num_experts), _p(idx), _p(ew), _p(cnt))
     return idx, ew, cnt
+
+
+def moe_align(topk_ids, num_experts: int) -> np.ndarray:
+    ids = _c(topk_ids, np.int32).ravel()
+    out = np.empty((num_experts, ids.size), np.int32)
+    lib().oracle_moe_align(_p(ids), I64(ids.size), I32(num_experts), _p(out))
+    return out
+
+
+def moe_align1(experts_info, topk_weights, experts_weight_info):
+    """In place on copies of the two tables -> (experts_info, experts_weight_info, expert_token_num)."""
+    info = np.array(experts_info, dtype=np.int32, order="C", copy=True)
+    wout = np.array(experts_weight_info, dtype=np.float32, order="C", copy=True)
+    w = _c(topk_weights, np.float32).ravel()
+    E, P = info.shape
+    assert w.size == P and wout.shape == info.shape
+    cnt = np.empty((E,), np.int32)
+    lib().oracle_moe_align1(_p(info), _p(w), I64(P), I32(E), _p(wout), _p(cnt))
+    return info, wout, cnt
 
 
 def moe_align2(num_pairs: int, expert_token_num, block_m: int) -> np.ndarray:

@@ -14,10 +14,11 @@
  * lives in tests/test_oracle_*.py):
  *   oracle_f32_to_e4m3fn        pinned: known-answer table + torch CPU cast over
  *                               every bf16 pattern and a dense fp32 sweep
- *   oracle_group_quant_fp8      pinned: torch closed form, special cases, invariants
+ *   oracle_group_quant_fp8(_f32) pinned: torch closed form (bf16, fp16 and fp32 inputs), special cases,
+ *                               invariants; groups holding NaN/Inf: own definition, outside the reference's contract
  *   oracle_block_weight_quant   pinned: torch closed form
  *   oracle_block_gemm*          pinned: unit-scale / one-hot special cases, numpy f64
- *   oracle_moe_align_fused/2    pinned: the reference's own golden vectors
+ *   oracle_moe_align, _align1, _align_fused, _align2   pinned: the reference's own golden vectors
  *   oracle_grouped_block_gemm   pinned: per-expert loop of the dense oracle
  *   oracle_silu_and_mul         pinned: torch closed form (bit-equal but for rare 1-ulp exp differences), special values
  *   oracle_moe_sum_reduce       pinned: exactly summable inputs, torch closed form
@@ -101,41 +102,69 @@ uint8_t oracle_f32_to_e4m3fn(float f) {
 
 /*
  * per_token_group_quant_fp8: one scale per `group` contiguous elements of a row.
- * Follows quantization/fp8act_quant_kernel.py:53-57 (kernel body) and :239-251
- * (the reference's own torch restatement):
+ * Follows quantization/fp8act_quant_kernel.py:52-57 (kernel body: any input dtype is
+ * widened to fp32 first, :52) and :239-251 (the reference's own torch restatement):
  *     y      = x.to(f32)
  *     absmax = max(max(|y|), eps)
  *     s      = absmax / 448           (IEEE division)
  *     q      = clamp(y / s, -448, 448).to(e4m3fn)
- * x: bf16 bit patterns [M,K] contiguous; q: bytes [M,K]; s: fp32 with element
- * strides (s_stride_m, s_stride_g) so both the row-major and the column-major
- * scale layouts (:37-42) are covered.
+ * x: fp32 values [M,K] contiguous (bf16 and fp16 inputs widen exactly); q: bytes
+ * [M,K]; s: fp32 with element strides (s_stride_m, s_stride_g) so both the
+ * row-major and the column-major scale layouts (:37-42) are covered.
+ *
+ * Non-finite inputs are outside the reference's contract (its max and clamp on NaN
+ * are unspecified).  This build defines them: a group that holds a NaN or an
+ * infinity gets the scale NaN (0x7FC00000) and every byte 0x7F with the sign bit of
+ * its element, so bad activations stay visible downstream instead of turning into
+ * plausible numbers.
  */
+static void group_quant_row(const float *xp, int32_t group, float eps, uint8_t *qp, float *sp) {
+    const float fp8_max = 448.0f;
+    float amax = 0.0f;
+    int finite = 1;
+    for (int32_t j = 0; j < group; ++j) {
+        float a = fabsf(xp[j]);
+        if (!(a <= 3.4028234663852886e38f)) finite = 0;   /* NaN or infinity */
+        if (a > amax) amax = a;
+    }
+    if (!finite) {
+        for (int32_t j = 0; j < group; ++j) qp[j] = (uint8_t)(((f32_to_bits(xp[j]) >> 24) & 0x80u) | 0x7fu);
+        *sp = bits_to_f32(0x7fc00000u);
+        return;
+    }
+    if (!(amax > eps)) amax = eps;
+    volatile float sc = amax / fp8_max;
+    for (int32_t j = 0; j < group; ++j) {
+        volatile float y = xp[j] / sc;
+        float c = y;
+        if (c > fp8_max) c = fp8_max;
+        if (c < -fp8_max) c = -fp8_max;
+        qp[j] = oracle_f32_to_e4m3fn(c);
+    }
+    *sp = sc;
+}
+
+void oracle_group_quant_fp8_f32(const float *x, int64_t M, int64_t K, int32_t group, float eps,
+                                uint8_t *q, float *s, int64_t s_stride_m, int64_t s_stride_g) {
+    int64_t G = K / group;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t g = 0; g < G; ++g)
+            group_quant_row(x + m * K + g * group, group, eps, q + m * K + g * group,
+                            s + m * s_stride_m + g * s_stride_g);
+}
+
+/* The same for bf16 bit patterns (the layout the hot path sees). */
 void oracle_group_quant_fp8(const uint16_t *x, int64_t M, int64_t K, int32_t group, float eps,
                             uint8_t *q, float *s, int64_t s_stride_m, int64_t s_stride_g) {
-    const float fp8_max = 448.0f;
     int64_t G = K / group;
-    for (int64_t m = 0; m < M; ++m) {
+    float *row = (float *)malloc((size_t)group * sizeof(float));
+    for (int64_t m = 0; m < M; ++m)
         for (int64_t g = 0; g < G; ++g) {
             const uint16_t *xp = x + m * K + g * group;
-            uint8_t *qp = q + m * K + g * group;
-            float amax = 0.0f;
-            for (int32_t j = 0; j < group; ++j) {
-                float a = fabsf(oracle_bf16_to_f32(xp[j]));
-                if (a > amax) amax = a;
-            }
-            if (!(amax > eps)) amax = eps;
-            volatile float sc = amax / fp8_max;
-            for (int32_t j = 0; j < group; ++j) {
-                volatile float y = oracle_bf16_to_f32(xp[j]) / sc;
-                float c = y;
-                if (c > fp8_max) c = fp8_max;
-                if (c < -fp8_max) c = -fp8_max;
-                qp[j] = oracle_f32_to_e4m3fn(c);
-            }
-            s[m * s_stride_m + g * s_stride_g] = sc;
+            for (int32_t j = 0; j < group; ++j) row[j] = oracle_bf16_to_f32(xp[j]);
+            group_quant_row(row, group, eps, q + m * K + g * group, s + m * s_stride_m + g * s_stride_g);
         }
-    }
+    free(row);
 }
 
 /*
@@ -263,6 +292,41 @@ void oracle_moe_align_fused(const int32_t *topk_ids, const float *topk_weights, 
         int32_t pos = expert_token_num[e]++;
         expert_to_token_index[(int64_t)e * num_pairs + pos] = (int32_t)i;
         expert_to_weight[(int64_t)e * num_pairs + pos] = topk_weights[i];
+    }
+}
+
+/*
+ * moe_align (grouped_fused_moe.py:39-98): 0/1 table [E, num_pairs], zero-filled first (:86), then 1 at
+ * (topk_ids[j], j) (:49-55).
+ */
+void oracle_moe_align(const int32_t *topk_ids, int64_t num_pairs, int32_t num_experts, int32_t *out) {
+    for (int64_t i = 0; i < (int64_t)num_experts * num_pairs; ++i) out[i] = 0;
+    for (int64_t j = 0; j < num_pairs; ++j) {
+        int32_t e = topk_ids[j];
+        if (e >= 0 && e < num_experts) out[(int64_t)e * num_pairs + j] = 1;
+    }
+}
+
+/*
+ * moe_align1 (grouped_fused_moe.py:101-214): for every expert, walk its row of the 0/1 table in order and
+ * write, IN PLACE, the position of each 1 at the next free slot (running count, :127-133), the weight of that
+ * pair at the same slot of experts_weight_info (:134-138), and the count (:140).  Slots past the count keep
+ * their old contents, which is what the reference's golden vector shows.
+ */
+void oracle_moe_align1(int32_t *experts_info, const float *topk_weights, int64_t num_pairs, int32_t num_experts,
+                       float *experts_weight_info, int32_t *expert_token_num) {
+    for (int32_t e = 0; e < num_experts; ++e) {
+        int32_t *row = experts_info + (int64_t)e * num_pairs;
+        float *wrow = experts_weight_info + (int64_t)e * num_pairs;
+        int32_t cnt = 0;
+        for (int64_t j = 0; j < num_pairs; ++j) {
+            if (row[j] == 1) {
+                row[cnt] = (int32_t)j;      /* cnt <= j: never overwrites an entry not yet visited */
+                wrow[cnt] = topk_weights[j];
+                ++cnt;
+            }
+        }
+        expert_token_num[e] = cnt;
     }
 }
 

@@ -100,3 +100,70 @@ def test_grouped_gemm_under_graph_capture(hip):
         return eager_out
 
     _replay_matches(eager, capture)
+
+
+def test_graph_survives_workspace_regrowth(hip):
+    """A graph captured at a split-K shape keeps the workspace address it was captured with.  A later eager call
+    that needs a larger workspace must not free that buffer: the replay afterwards still has to give the eager
+    result, and so does the large call."""
+    from lightllm_amd import _lib
+    from lightllm_amd.quantization import per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    print("graph capture across workspace regrowth", flush=True)
+    M, N, K = 8, 4096, 14336                      # stream kernel, K split over CTAs: uses partials + counters
+    xq, xs = per_token_group_quant_fp8(H.activations(M, K, seed=31).cuda(), 128)
+    wq, ws = H.quantized_weights(N, K, seed=32, device="cuda")
+    expect = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), expect, [128, 128])
+    torch.cuda.synchronize()
+
+    out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128])
+        torch.cuda.synchronize()
+        first_ws = _lib.workspace(xq.device, 1)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128])
+        # a call on the same stream that outgrows the workspace, then garbage written wherever the allocator
+        # would have recycled a freed buffer
+        bigger = _lib.workspace(xq.device, first_ws.numel() + (8 << 20))
+        assert bigger.data_ptr() != first_ws.data_ptr()
+        del first_ws
+        junk = [torch.full((first_n,), 0x7F, dtype=torch.uint8, device="cuda") for first_n in (33 << 20, 33 << 20)]
+        torch.cuda.synchronize()
+        for r in range(3):
+            out.fill_(float("nan"))
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), expect.view(torch.int16)), f"replay {r}"
+            eager = torch.empty_like(out)
+            w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), eager, [128, 128])   # now on the larger workspace
+            torch.cuda.synchronize()
+            assert torch.equal(eager.view(torch.int16), expect.view(torch.int16))
+        del junk
+    torch.cuda.current_stream().wait_stream(side)
+
+
+def test_reset_workspace_recovers_dirty_counters(hip):
+    """Counter words left non-zero (as an aborted launch would) make a split-K launch wrong; the reset entry point
+    restores the invariant."""
+    from lightllm_amd import _lib
+    from lightllm_amd.quantization import per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    M, N, K = 8, 4096, 14336
+    xq, xs = per_token_group_quant_fp8(H.activations(M, K, seed=33).cuda(), 128)
+    wq, ws = H.quantized_weights(N, K, seed=34, device="cuda")
+    expect = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), expect, [128, 128])
+    torch.cuda.synchronize()
+    buf = _lib.workspace(xq.device, 1)
+    buf[: _lib.WS_COUNTER_BYTES].view(torch.int32).fill_(1 << 20)   # no CTA will ever see itself as the last arrival
+    _lib.reset_workspace(xq.device)
+    out = torch.empty_like(expect)
+    w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128])
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), expect.view(torch.int16))
+    assert int(buf[: _lib.WS_COUNTER_BYTES].view(torch.int32).abs().max()) == 0

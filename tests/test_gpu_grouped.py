@@ -52,6 +52,42 @@ def test_moe_align_fused_reference_vectors(hip):
     _check_align(ids, torch.arange(ids.numel(), dtype=torch.float32).reshape(5121, 8), 257)
 
 
+def test_moe_align_and_align1_reference_vectors(hip):
+    """Golden vectors of the reference's test_moe_align / test_moe_align1 (test_grouped_fused_moe.py:26-77), then
+    the two-step form against the oracle at sizes that span several 4096-pair steps and every padding."""
+    import oracle
+    from lightllm_amd.fused_moe import moe_align, moe_align1
+
+    print("moe_align / moe_align1", flush=True)
+    ids = torch.tensor([[0, 1, 2], [0, 3, 1], [3, 1, 4]], dtype=torch.int32, device="cuda")
+    out = torch.full((5, 9), 7, dtype=torch.int32, device="cuda")
+    moe_align(ids, out)
+    assert out.cpu().tolist() == [
+        [1, 0, 0, 1, 0, 0, 0, 0, 0], [0, 1, 0, 0, 0, 1, 0, 1, 0], [0, 0, 1, 0, 0, 0, 0, 0, 0],
+        [0, 0, 0, 0, 1, 0, 1, 0, 0], [0, 0, 0, 0, 0, 0, 0, 0, 1]]
+    info = torch.tensor([[1, 0, 0, 0], [0, 1, 1, 0], [0, 0, 0, 1], [0, 0, 0, 0]], dtype=torch.int32, device="cuda")
+    tw = torch.tensor([[0.3, 0.7], [0.2, 0.8]], dtype=torch.float32, device="cuda")
+    cnt = torch.zeros((4,), dtype=torch.int32, device="cuda")
+    wout = torch.zeros((4, 4), dtype=torch.float32, device="cuda")
+    moe_align1(info, tw, wout, cnt, 2)
+    assert cnt.cpu().tolist() == [1, 2, 1, 0]
+    assert info.cpu().tolist() == [[0, 0, 0, 0], [1, 2, 1, 0], [3, 0, 0, 1], [0, 0, 0, 0]]
+    assert torch.allclose(wout.cpu(), torch.tensor([[0.3, 0, 0, 0], [0.7, 0.2, 0, 0], [0.8, 0, 0, 0], [0, 0, 0, 0]]))
+    for (T, E, topk, seed) in [(1, 3, 2, 1), (300, 12, 4, 2), (5121, 257, 8, 3), (4097, 2, 1, 4)]:
+        ids_c, tw_c = H.routing(T, E, topk, seed=seed)
+        mask = torch.empty((E, T * topk), dtype=torch.int32, device="cuda")
+        moe_align(ids_c.cuda(), mask)
+        mask_ref = oracle.moe_align(ids_c.numpy(), E)
+        assert np.array_equal(mask.cpu().numpy(), mask_ref)
+        wout = torch.zeros((E, T * topk), dtype=torch.float32, device="cuda")
+        cnt = torch.empty((E,), dtype=torch.int32, device="cuda")
+        moe_align1(mask, tw_c.cuda(), wout, cnt, topk)
+        info_ref, w_ref, cnt_ref = oracle.moe_align1(mask_ref, tw_c.numpy(), np.zeros(mask_ref.shape, np.float32))
+        assert np.array_equal(cnt.cpu().numpy(), cnt_ref)
+        assert np.array_equal(mask.cpu().numpy(), info_ref)          # in place, tails included
+        assert np.array_equal(wout.cpu().numpy(), w_ref)
+
+
 def test_moe_align2_reference_vectors(hip):
     """Golden vectors of the reference's test_moe_align2 (test_grouped_fused_moe.py:219-258)."""
     from lightllm_amd.fused_moe import moe_align2

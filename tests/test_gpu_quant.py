@@ -125,3 +125,52 @@ def test_preconditions(hip):
         per_token_group_quant_fp8(torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")[:, ::2], 64)
     xq, xs = per_token_group_quant_fp8(torch.zeros((0, 256), dtype=torch.bfloat16, device="cuda"), 128)
     assert xq.shape == (0, 256) and xs.shape == (0, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K", [(1, 128), (33, 384), (257, 7168), (64, 14336)])
+def test_bit_exact_fp16_fp32_activations(hip, dtype, M, K):
+    """The reference widens any input dtype to fp32 (fp8act_quant_kernel.py:52); so does the oracle."""
+    print(f"quant {dtype} M={M} K={K}", flush=True)
+    g = H.gen(M * 7 + K)
+    x = torch.randn((M, K), generator=g, dtype=torch.float32)
+    x[:, ::97] *= 37.0
+    if M > 1:
+        x[1] = 0.0
+    x = x.to(dtype)
+    xq, xs = _run(x)
+    q_ref, s_ref = oracle.group_quant_fp8_f32(x.float().numpy())
+    assert np.array_equal(tr.bits_of(xs.contiguous()), s_ref.view(np.uint32))
+    assert np.array_equal(tr.bits_of(xq), q_ref)
+
+
+def test_fp32_wide_dynamic_range(hip):
+    """fp32 groups spanning subnormals to 1e38, and values that are not bf16-representable."""
+    g = H.gen(21)
+    M, K = 256, 1024
+    expo = torch.randint(-140, 120, (M, K // 128, 1), generator=g).float()
+    x = (torch.randn((M, K // 128, 128), generator=g) * torch.exp2(expo)).reshape(M, K).contiguous()
+    xq, xs = _run(x)
+    q_ref, s_ref = oracle.group_quant_fp8_f32(x.numpy())
+    assert np.array_equal(tr.bits_of(xs.contiguous()), s_ref.view(np.uint32))
+    assert np.array_equal(tr.bits_of(xq), q_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_non_finite_groups_are_poisoned(hip, dtype):
+    """One NaN, one +Inf and one -Inf group among finite ones: scale NaN, bytes 0x7F | sign; the finite groups
+    of the same rows are untouched (the reference leaves this case undefined; the oracle states this build's rule)."""
+    x = H.activations(8, 512, seed=13).float()
+    x[1, 130] = float("nan")
+    x[2, 5] = float("inf")
+    x[3, 300] = float("-inf")
+    x[4, 384] = float("nan")
+    x[4, 385] = float("inf")
+    x = x.to(dtype)
+    xq, xs = _run(x)
+    q_ref, s_ref = oracle.group_quant_fp8_f32(x.float().numpy())
+    q, s = tr.bits_of(xq), tr.bits_of(xs.contiguous())
+    assert np.array_equal(q, q_ref)
+    assert np.array_equal(s, s_ref.view(np.uint32))
+    assert s[1, 1] == 0x7FC00000 and s[2, 0] == 0x7FC00000 and s[3, 2] == 0x7FC00000 and s[4, 3] == 0x7FC00000
+    assert np.all((q[1, 128:256] & 0x7F) == 0x7F) and np.all((q[1, :128] & 0x7F) != 0x7F)

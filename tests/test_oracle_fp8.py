@@ -357,3 +357,144 @@ def test_fused_experts_composition_against_dense_float():
             want[t] += tw[t, k] * (a @ d2.T)
     assert tr.cosine(got, want) > 0.999
     assert (got - want).abs().max() / want.abs().max() < 0.05
+
+
+# ---- activation quantizer: other input dtypes, non-finite groups ---------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+def test_group_quant_f32_entry_equals_torch_closed_form(dtype):
+    """The reference widens any input to fp32 first (fp8act_quant_kernel.py:52); torch's closed form does the same."""
+    g = H.gen(91)
+    x = (torch.randn((48, 1024), generator=g) * torch.exp2(torch.randint(-12, 12, (48, 8, 1), generator=g).float())
+         .repeat_interleave(128, -1).reshape(48, 1024)).to(dtype)
+    x[5] = 0.0
+    q_t, s_t = tr.group_quant(x)
+    q_c, s_c = oracle.group_quant_fp8_f32(x.float().numpy())
+    assert np.array_equal(tr.bits_of(s_t), s_c.view(np.uint32))
+    assert np.array_equal(tr.bits_of(q_t), q_c)
+    if dtype == torch.bfloat16:
+        q_b, s_b = oracle.group_quant_fp8(tr.bits_of(x))
+        assert np.array_equal(q_b, q_c) and np.array_equal(s_b.view(np.uint32), s_c.view(np.uint32))
+
+
+def test_group_quant_non_finite_groups_follow_the_stated_rule():
+    """Outside the reference's contract.  The rule of this build: a group holding NaN or +-Inf gets scale NaN and
+    bytes 0x7F | sign; the other groups of the row are quantized as usual."""
+    x = H.activations(4, 384, seed=92).float()
+    clean_q, clean_s = oracle.group_quant_fp8_f32(x.numpy())
+    x[0, 3] = float("nan")
+    x[1, 200] = float("inf")
+    x[2, 383] = float("-inf")
+    q, s = oracle.group_quant_fp8_f32(x.numpy())
+    su = s.view(np.uint32)
+    assert su[0, 0] == 0x7FC00000 and su[1, 1] == 0x7FC00000 and su[2, 2] == 0x7FC00000
+    neg = (x.numpy().view(np.uint32) >> 31).astype(np.uint8)
+    for (r, g) in [(0, 0), (1, 1), (2, 2)]:
+        sl = slice(128 * g, 128 * g + 128)
+        assert np.array_equal(q[r, sl], 0x7F | (neg[r, sl] << 7))
+    keep = np.ones((4, 3), bool)
+    keep[0, 0] = keep[1, 1] = keep[2, 2] = False
+    assert np.array_equal(su[keep], clean_s.view(np.uint32)[keep])
+    assert np.array_equal(q.reshape(4, 3, 128)[keep], clean_q.reshape(4, 3, 128)[keep])
+    assert np.array_equal(q[3], clean_q[3])
+
+
+def test_fused_experts_composition_is_exact_when_every_step_is():
+    """Integer payloads and power-of-two scales make both GEMMs exact, so the only inexact steps left are the
+    SiLU (checked value by value against float64 here) and the group quantizer of its output (torch's closed
+    form).  A float64 evaluation with the reference's rounding points
+    (fused_moe/grouped_fused_moe.py:1048-1113: bf16 after each GEMM and after silu_and_mul, fp32 sum over the
+    slots in ascending order) must then equal the oracle bit for bit."""
+    T, Hd, I, E, topk = 10, 256, 256, 5, 2
+    g = H.gen(93)
+    # activations: small integers, one 448 per group so that every activation scale is exactly 1
+    x = torch.randint(-2, 3, (T, Hd), generator=g).float()
+    x[:, ::128] = 448.0
+    x_b = x.to(torch.bfloat16)
+    xq_t, xs_t = tr.group_quant(x_b)
+    assert torch.all(xs_t == 1.0) and torch.equal(xq_t.float(), x)
+    # weights: sparse {-1, 0, 1} payloads (zero against the 448 columns), power-of-two block scales
+    def payload(*shape):
+        w = torch.randint(-1, 2, shape, generator=g).float() * (torch.rand(shape, generator=g) < 0.25)
+        return w
+    w1 = payload(E, 2 * I, Hd)
+    w1[:, :, ::128] = 0.0
+    w2 = payload(E, Hd, I)
+    w1_s = torch.exp2(torch.randint(-2, 2, (E, 2 * I // 128, Hd // 128), generator=g).float())
+    w2_s = torch.exp2(torch.randint(-3, 1, (E, Hd // 128, I // 128), generator=g).float())
+    w1_q, w2_q = w1.to(torch.float8_e4m3fn), w2.to(torch.float8_e4m3fn)
+    ids, tw = H.routing(T, E, topk, seed=94)
+    # routed weights with few mantissa bits keep the last product exact enough to be rounded once
+    tw = (tw * 16).round().clamp_min(1) / 16
+
+    out = oracle.fused_experts(tr.bits_of(x_b), tr.bits_of(w1_q), w1_s.numpy(), tr.bits_of(w2_q), w2_s.numpy(),
+                               ids.numpy(), tw.numpy())
+    got = tr.bf16_from_bits(out)
+
+    d1 = (w1.double().reshape(E, 2 * I // 128, 128, Hd // 128, 128) * w1_s.double()[:, :, None, :, None]).reshape(E, 2 * I, Hd)
+    slots = torch.zeros((T, topk, Hd), dtype=torch.bfloat16)
+    seen_gate = set()
+    for t in range(T):
+        for k in range(topk):
+            e = int(ids[t, k])
+            h1 = (d1[e] @ x.double()[t])                      # exact: integers times powers of two
+            h1_b = h1.to(torch.bfloat16)
+            assert torch.equal(h1_b.double(), h1), "first GEMM must be exact in bf16 for this test"
+            gate, up = h1_b[:I].double(), h1_b[I:].double()
+            seen_gate.update(gate.tolist())
+            act = ((gate / (1.0 + torch.exp(-gate))).to(torch.bfloat16).double() * up).to(torch.bfloat16)
+            aq, asc = tr.group_quant(act.reshape(1, I))
+            acc = torch.zeros(Hd, dtype=torch.float64)
+            for kb in range(I // 128):
+                dot = w2[e][:, 128 * kb:128 * kb + 128].double() @ aq[0, 128 * kb:128 * kb + 128].double()
+                acc = (acc.float() + (dot * asc[0, kb].double()).float() *
+                       w2_s[e, :, kb].repeat_interleave(128).float()).double()   # fp32 running sum per block
+            slots[t, k] = (acc.float() * tw[t, k]).to(torch.bfloat16)
+    # the oracle's SiLU (libm expf in fp32) against float64 on every gate value that occurred
+    gv = torch.tensor(sorted(seen_gate), dtype=torch.float64)
+    pair = torch.stack([gv, torch.ones_like(gv)], 0).reshape(1, -1).to(torch.bfloat16)   # [gate | up = 1]
+    silu_c = tr.bf16_from_bits(oracle.silu_and_mul(tr.bits_of(pair.reshape(1, 2 * gv.numel()))))
+    assert torch.equal(silu_c[0].double(), (gv / (1.0 + torch.exp(-gv))).to(torch.bfloat16).double())
+    want = slots.float().sum(dim=1) if topk == 1 else None
+    acc = torch.zeros((T, Hd), dtype=torch.float32)
+    for k in range(topk):
+        acc += slots[:, k].float()
+    want = acc.to(torch.bfloat16)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+# ---- the two-step routing tables (moe_align, moe_align1) ------------------------------------------------------
+MOE_ALIGN_IDS = [[0, 1, 2], [0, 3, 1], [3, 1, 4]]
+MOE_ALIGN_GOLD = [  # unit_tests/common/fused_moe/test_grouped_fused_moe.py:26-47
+    [1, 0, 0, 1, 0, 0, 0, 0, 0],
+    [0, 1, 0, 0, 0, 1, 0, 1, 0],
+    [0, 0, 1, 0, 0, 0, 0, 0, 0],
+    [0, 0, 0, 0, 1, 0, 1, 0, 0],
+    [0, 0, 0, 0, 0, 0, 0, 0, 1],
+]
+MOE_ALIGN1_INFO = [[1, 0, 0, 0], [0, 1, 1, 0], [0, 0, 0, 1], [0, 0, 0, 0]]
+MOE_ALIGN1_W = [[0.3, 0.7], [0.2, 0.8]]
+MOE_ALIGN1_GOLD_INFO = [[0, 0, 0, 0], [1, 2, 1, 0], [3, 0, 0, 1], [0, 0, 0, 0]]   # same file :50-77
+MOE_ALIGN1_GOLD_W = [[0.3, 0, 0, 0], [0.7, 0.2, 0, 0], [0.8, 0, 0, 0], [0, 0, 0, 0]]
+MOE_ALIGN1_GOLD_CNT = [1, 2, 1, 0]
+
+
+def test_moe_align_reference_golden():
+    out = oracle.moe_align(np.array(MOE_ALIGN_IDS, np.int32), 5)
+    assert out.tolist() == MOE_ALIGN_GOLD
+
+
+def test_moe_align1_reference_golden():
+    info, w, cnt = oracle.moe_align1(MOE_ALIGN1_INFO, MOE_ALIGN1_W, np.zeros((4, 4), np.float32))
+    assert info.tolist() == MOE_ALIGN1_GOLD_INFO
+    assert cnt.tolist() == MOE_ALIGN1_GOLD_CNT
+    assert np.allclose(w, np.array(MOE_ALIGN1_GOLD_W, np.float32))
+
+
+def test_moe_align_then_align1_equals_the_fused_form():
+    ids, tw = H.routing(300, 12, 4, seed=95)
+    mask = oracle.moe_align(ids.numpy(), 12)
+    info, w, cnt = oracle.moe_align1(mask, tw.numpy(), np.zeros(mask.shape, np.float32))
+    idx_f, w_f, cnt_f = oracle.moe_align_fused(ids.numpy(), tw.numpy(), 12)
+    assert np.array_equal(cnt, cnt_f)
+    for e in range(12):
+        assert np.array_equal(info[e, :cnt[e]], idx_f[e, :cnt[e]]) and np.array_equal(w[e, :cnt[e]], w_f[e, :cnt[e]])
