@@ -31,6 +31,7 @@ extern "C" {
 #define MI355_EWORKSPACE -4    /* workspace missing or smaller than *_workspace_bytes() */
 #define MI355_ELAUNCH -5       /* the HIP runtime refused the launch (hipLaunchKernel / hipFuncSetAttribute failed) */
 #define MI355_EUNSUPPORTED -6  /* valid request that no kernel variant covers */
+#define MI355_ESCRATCH -7      /* mi355_block_fp8_gemm_noalloc: the launch needs more scratch than the library holds */
 
 const char *mi355_error_string(int code);
 
@@ -114,6 +115,21 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
 
 /* Bytes of workspace the launch plan of the CURRENT device needs for this shape and variant (0 = none). */
 size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant);
+
+/* mi355_block_fp8_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as
+ * mi355_block_fp8_gemm without the workspace pair: split-K partials and counters go to a fixed array inside the
+ * library's device image, MI355_WS_COUNTER_BYTES + MI355_NOALLOC_PARTIAL_MIB MiB per GPU, held from the first call
+ * on that GPU until the process ends.  A launch plan that needs more returns MI355_ESCRATCH and launches nothing
+ * (mi355_block_fp8_gemm_workspace_bytes() tells the need).  The call allocates and frees nothing; it clears the
+ * counter words with a small fill kernel first.  All calls on one GPU share the array: calls that may overlap on
+ * one GPU (different streams, concurrently replayed graphs) race - use mi355_block_fp8_gemm with one workspace per
+ * stream there. */
+#define MI355_NOALLOC_PARTIAL_MIB 8
+int mi355_block_fp8_gemm_noalloc(const void *A, const void *B, const float *As, const float *Bs, void *C, int64_t M,
+                                 int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                                 int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int32_t block_n,
+                                 int32_t block_k, int32_t variant, void *stream);
 
 /* Re-zeroes the MI355_WS_COUNTER_BYTES counter bytes of a workspace (a small fill kernel on `stream`).  The
  * kernels leave the counters zero themselves; this is the recovery path after a launch that was aborted, or

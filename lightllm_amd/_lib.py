@@ -23,6 +23,11 @@ SIGNATURES = {
     "mi355_group_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _f32, _i64, _i64, _vp]),
     "mi355_block_weight_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp]),
     "mi355_block_fp8_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "mi355_block_fp8_gemm_noalloc": (
+        _c.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
+         _i32, _vp],
+    ),
     "mi355_reset_workspace": (_c.c_int, [_vp, _sz, _vp]),
     "mi355_block_fp8_gemm": (
         _c.c_int,
@@ -83,7 +88,7 @@ def check(code: int, what: str) -> None:
     msg = lib().mi355_error_string(code).decode()
     if code in (-2,):
         raise AssertionError(f"{what}: {msg}")
-    if code in (-1, -3, -4, -6):
+    if code in (-1, -3, -4, -6, -7):
         raise ValueError(f"{what}: {msg}")
     raise Mi355Error(f"{what}: {msg}")
 

@@ -332,6 +332,51 @@ __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, uint32_t n
 
 }  // namespace mi355
 
+// ---- the entry point that allocates nothing -------------------------------------------------------------
+// Split-K partials, arrival counters and the tile counters of the persistent launch live in a fixed array in
+// the library's own device image instead of a caller-owned workspace.  Every GPU holds its own copy of the
+// array at its own address; in host code the array's name is only a handle for hipGetSymbolAddress.
+namespace mi355 {
+
+constexpr size_t kScratchBytes = (size_t)MI355_WS_COUNTER_BYTES + ((size_t)MI355_NOALLOC_PARTIAL_MIB << 20);
+static __device__ __align__(256) uint8_t scratch[kScratchBytes];
+
+// Device address of `scratch` on the current device, looked up on the first call per device.
+static void *scratch_ptr() {
+    static std::atomic<void *> ptrs[kMaxDevices];
+    const int dev = current_device();
+    if (dev < 0 || dev >= kMaxDevices) return nullptr;
+    void *p = ptrs[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+    ptrs[dev].store(p, std::memory_order_release);
+    return p;
+}
+
+}  // namespace mi355
+
+extern "C" int mi355_block_fp8_gemm_noalloc(const void *A, const void *B, const float *As, const float *Bs, void *C,
+                                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
+                                            int64_t ldb_n, int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k,
+                                            int64_t bs_n, int32_t block_n, int32_t block_k, int32_t variant,
+                                            void *stream) {
+    const size_t need = mi355_block_fp8_gemm_workspace_bytes(M, N, K, variant);
+    if (need > kScratchBytes) return MI355_ESCRATCH;
+    void *ws = nullptr;
+    if (need > 0) {
+        ws = scratch_ptr();
+        if (!ws) return MI355_ELAUNCH;
+        // The array keeps what the last call left.  The kernels need their counter words zero and leave them
+        // zero, but a launch that was aborted would not have: clear them here (a fill kernel, not a memset node,
+        // so that the call can be captured into a HIP graph).
+        const uint32_t words = MI355_WS_COUNTER_BYTES / 4;
+        const int rc = launch(zero_words_kernel, dim3(words / 256), dim3(256), 0, (hipStream_t)stream, (uint32_t *)ws, words);
+        if (rc != MI355_OK) return rc;
+    }
+    return mi355_block_fp8_gemm(A, B, As, Bs, C, M, N, K, lda, ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n, block_n,
+                                block_k, ws, ws ? kScratchBytes : 0, variant, stream);
+}
+
 /* Re-zeroes the counter words of a caller-owned workspace (recovery after an aborted launch). */
 extern "C" int mi355_reset_workspace(void *ws, size_t ws_bytes, void *stream) {
     if (!ws || ws_bytes < (size_t)MI355_WS_COUNTER_BYTES || ((uintptr_t)ws & 3)) return MI355_EWORKSPACE;

@@ -11,6 +11,7 @@ extern "C" const char *mi355_error_string(int code) {
         case MI355_EWORKSPACE: return "workspace missing, misaligned or too small";
         case MI355_ELAUNCH: return "HIP runtime refused the launch";
         case MI355_EUNSUPPORTED: return "no kernel variant covers this request";
+        case MI355_ESCRATCH: return "the launch needs more scratch than the no-allocation entry point holds";
         default: return "unknown error code";
     }
 }
