@@ -28,8 +28,9 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def _time_calls(fn, iters, warm):
-    """Average duration of `fn` in microseconds, HIP events on torch's current stream (the launch stream)."""
+def _time_calls(fn, iters, warm, batches=7):
+    """Duration of `fn` in microseconds: the median over `batches` back-to-back batches of `iters` calls, each
+    batch bracketed by HIP events on torch's current stream (the launch stream)."""
     import torch
 
     # sustained load first: the clocks need tens of milliseconds to settle after an idle gap
@@ -41,13 +42,32 @@ def _time_calls(fn, iters, warm):
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
-    s, e = _events(2)
-    s.record()
-    for _ in range(iters):
-        fn()
-    e.record()
+    ev = _events(batches + 1)
+    ev[0].record()
+    for b in range(batches):
+        for _ in range(iters):
+            fn()
+        ev[b + 1].record()
     torch.cuda.synchronize()
-    return s.elapsed_time(e) * 1e3 / iters
+    per_call = sorted(ev[b].elapsed_time(ev[b + 1]) * 1e3 / iters for b in range(batches))
+    return per_call[batches // 2]
+
+
+def _rotating(items):
+    """Calls see `items` round-robin, so that a bandwidth-bound launch never finds its input in the 256 MB
+    memory-side cache left there by the previous launch."""
+    state = [0]
+
+    def nxt():
+        it = items[state[0] % len(items)]
+        state[0] += 1
+        return it
+
+    return nxt
+
+
+def roofline_us(flops, nbytes):
+    return max(nbytes / HBM_PEAK_GBS / 1e3, flops / FP8_MFMA_PEAK_TFLOPS / 1e6)
 
 
 def gemm_bytes(M, N, K):
@@ -184,7 +204,8 @@ def main():
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
         ms_per_step = elapsed * 1e3 / args.steps
-        gemm_us = sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(args.steps)) * 1e3 / args.steps
+        gemm_all = sorted(ev[2 * i].elapsed_time(ev[2 * i + 1]) * 1e3 for i in range(args.steps))
+        gemm_us = gemm_all[len(gemm_all) // 2]   # median launch duration
         flops = 2.0 * M * N * K
         value = flops / (ms_per_step * 1e-3) / 1e12
         achieved = flops / (gemm_us * 1e-6) / 1e12
@@ -219,6 +240,7 @@ def main():
                 "traffic": 2.0043e9,
                 "algorithmic_bytes_per_launch": gemm_bytes(M, N, K),
                 "launch_us": round(gemm_us, 2),
+                "launch_us_min_max": [round(gemm_all[0], 2), round(gemm_all[-1], 2)],
                 "algorithmic_flops_per_launch": flops,
                 "peak_derived_from_device": round(derived_peak, 1),
             },
@@ -227,56 +249,79 @@ def main():
         torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "quant":
-        # standalone quantizer bandwidth test: [16384,7168] with 1% x50 outliers and an all-zero row
+        # standalone quantizer bandwidth test: [16384,7168] with 1% x50 outliers and an all-zero row; the input
+        # rotates through 4 distinct tensors (940 MB) and the outputs through 4 more
         Mq, Kq = 16384, 7168
-        x = make_act(Mq, Kq, 4, dev, outliers=True)
-        xq = torch.empty((Mq, Kq), dtype=torch.float8_e4m3fn, device=dev)
-        xs = torch.empty((Mq, Kq // 128), dtype=torch.float32, device=dev)
-        us = _time_calls(lambda: lightllm_per_token_group_quant_fp8(x, 128, xq, xs), 50, 5)
+        sets = []
+        for c in range(4):
+            sets.append((make_act(Mq, Kq, 4 + c, dev, outliers=True),
+                         torch.empty((Mq, Kq), dtype=torch.float8_e4m3fn, device=dev),
+                         torch.empty((Mq, Kq // 128), dtype=torch.float32, device=dev)))
+        nxt = _rotating(sets)
+
+        def call():
+            x, xq, xs = nxt()
+            lightllm_per_token_group_quant_fp8(x, 128, xq, xs)
+
+        us = _time_calls(call, 20, 5)
         gbs = quant_bytes(Mq, Kq) / us / 1e3
         others.append({"name": "per_token_group_quant_fp8 [16384,7168]", "us": round(us, 2), "GB/s": round(gbs, 1),
-                       "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
-        del x, xq, xs
+                       "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "rotated_MB": round(4 * Mq * Kq * 2 / 1e6)})
+        del sets, nxt
         torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "decode":
-        # Llama-3-8B decode linears; weights rotate through 5 copies so that no launch finds them in the
-        # 256 MB memory-side cache
+        # Llama-3-8B decode linears; the weights rotate through enough copies (> 600 MB) that no launch finds them
+        # in the 256 MB memory-side cache
         for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down")]:
-            copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(5)]
+            ncopies = -(-640_000_000 // (Nd * Kd))
+            copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(ncopies)]
+            views = [(q.t(), s.t()) for q, s in copies]
             for Md in (1, 8, 32, 64):
                 xq, xs = per_token_group_quant_fp8(make_act(Md, Kd, 20 + Md, dev), 128)
                 out = torch.empty((Md, Nd), dtype=torch.bfloat16, device=dev)
-                idx = [0]
+                nxt = _rotating(views)
 
                 def call():
-                    q, s = copies[idx[0] % 5]
-                    idx[0] += 1
-                    w8a8_block_fp8_matmul(xq, q.t(), xs, s.t(), out, [128, 128])
+                    q_t, s_t = nxt()
+                    w8a8_block_fp8_matmul(xq, q_t, xs, s_t, out, [128, 128])
 
-                us = _time_calls(call, 40, 10)
+                us = _time_calls(call, 2 * ncopies, ncopies)
                 gbs = gemm_bytes(Md, Nd, Kd) / us / 1e3
                 others.append({"name": f"llama3-8b {name} M={Md} N={Nd} K={Kd}", "us": round(us, 2),
                                "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
-                               "TFLOP/s": round(2.0 * Md * Nd * Kd / us / 1e6, 2)})
-            del copies
+                               "TFLOP/s": round(2.0 * Md * Nd * Kd / us / 1e6, 2),
+                               "rotated_MB": round(ncopies * Nd * Kd / 1e6)})
+            del copies, views
             torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "prefill":
-        for (Np, Kp, name) in [(7168, 18432, "down"), (2112, 7168, "q_a+kv_a")]:
+        # the three DeepSeek-V3 prefill linears over M (the shape -> variant table has two thresholds), and one K
+        # that is not a multiple of 1024 (q_b: K=1536); each row against its own roofline
+        # max(bytes / 8 TB/s, flops / 5.03 PFLOP/s)
+        shapes = [(36864, 7168, "gate_up"), (7168, 18432, "down"), (2112, 7168, "q_a+kv_a"), (24576, 1536, "q_b")]
+        for (Np, Kp, name) in shapes:
             wq, ws = make_weight(Np, Kp, 30, dev)
-            xq, xs = per_token_group_quant_fp8(make_act(M, Kp, 31, dev), 128)
-            out = torch.empty((M, Np), dtype=torch.bfloat16, device=dev)
-            us = _time_calls(lambda: w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128]), 20, 5)
-            tf = 2.0 * M * Np * Kp / us / 1e6
-            others.append({"name": f"deepseek-v3 {name} M=4096 N={Np} K={Kp}", "us": round(us, 2),
-                           "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / FP8_MFMA_PEAK_TFLOPS, 4)})
-            del wq, ws, xq, xs, out
+            wq_t, ws_t = wq.t(), ws.t()
+            for Mp in (128, 256, 512, 1024, 2048, 4096):
+                if name == "gate_up" and Mp == 4096:
+                    continue  # the headline
+                xq, xs = per_token_group_quant_fp8(make_act(Mp, Kp, 31, dev), 128)
+                out = torch.empty((Mp, Np), dtype=torch.bfloat16, device=dev)
+                us = _time_calls(lambda: w8a8_block_fp8_matmul(xq, wq_t, xs, ws_t, out, [128, 128]), 10, 3, batches=5)
+                flops = 2.0 * Mp * Np * Kp
+                tf = flops / us / 1e6
+                roof = roofline_us(flops, gemm_bytes(Mp, Np, Kp))
+                others.append({"name": f"deepseek-v3 {name} M={Mp} N={Np} K={Kp}", "us": round(us, 2),
+                               "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / FP8_MFMA_PEAK_TFLOPS, 4),
+                               "roofline_us": round(roof, 2), "frac_roofline": round(roof / us, 4)})
+                del xq, xs, out
+            del wq, ws, wq_t, ws_t
             torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "grouped":
-        # routed experts: 4096 tokens x top-8 over 256 experts, Zipf(1.1) popularity; weights are random fp8
-        # bytes here (11.3 GB; values do not change the timing), scales uniform in [0.5, 1.5) * 2e-4
+        # routed experts: 4096 tokens x top-8 over 256 experts, Zipf(1.1) popularity; weights ~N(0, 0.02) bf16,
+        # block-quantized expert by expert by the library's load-time quantizer (11.3 GB of e4m3 bytes)
         T, E, topk = 4096, 256, 8
         g = torch.Generator(device=dev).manual_seed(5)
         perm = torch.randperm(E, generator=g, device=dev)
@@ -291,22 +336,29 @@ def main():
         moe_align_fused(e2t, e2w, cnt, ids, tw)
         experts_hit = int((cnt > 0).sum())
 
-        def rand_fp8(shape):
-            b = torch.randint(0, 256, shape, dtype=torch.uint8, device=dev, generator=g)
-            return (b & 0xB7).view(torch.float8_e4m3fn)  # clears one exponent and one mantissa bit: no NaN codes
+        def expert_weights(Ng, Kg):
+            from lightllm_amd.quantization import mm_weight_quant
+
+            w = torch.empty((E, Ng, Kg), dtype=torch.float8_e4m3fn, device=dev)
+            sc = torch.empty((E, Ng // 128, Kg // 128), dtype=torch.float32, device=dev)
+            for e in range(E):
+                wb = (torch.randn((Ng, Kg), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16)
+                w[e], sc[e] = mm_weight_quant(wb)
+            return w, sc
 
         for (Ng, Kg, tk, mulw, name) in [(4096, 7168, topk, False, "gate_up"), (7168, 2048, 1, True, "down")]:
-            w = rand_fp8((E, Ng, Kg))
-            wscale = (torch.rand((E, Ng // 128, Kg // 128), generator=g, device=dev) + 0.5) * 2e-4
+            w, wscale = expert_weights(Ng, Kg)
             rows = T if tk == topk else P
             xq, xs = per_token_group_quant_fp8(make_act(rows, Kg, 40, dev), 128)
             out = torch.empty((P, Ng), dtype=torch.bfloat16, device=dev)
-            us = _time_calls(lambda: grouped_matmul(P, xq, xs, cnt, e2t, e2w, w, wscale, tk, out, mulw, True), 10, 3)
+            us = _time_calls(lambda: grouped_matmul(P, xq, xs, cnt, e2t, e2w, w, wscale, tk, out, mulw, True), 5, 3,
+                             batches=5)
             flops = 2.0 * P * Ng * Kg
             byts = experts_hit * Ng * Kg + rows * Kg + 2 * P * Ng
+            roof = roofline_us(flops, byts)
             others.append({"name": f"deepseek-v3 routed experts {name}: {P} rows, E={E}, N={Ng} K={Kg}",
                            "us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1), "GB/s": round(byts / us / 1e3, 1),
-                           "roofline_us": round(max(byts / HBM_PEAK_GBS / 1e3, flops / FP8_MFMA_PEAK_TFLOPS / 1e6), 1),
+                           "roofline_us": round(roof, 1), "frac_roofline": round(roof / us, 4),
                            "experts_hit": experts_hit})
             del w, wscale, xq, xs, out
             torch.cuda.empty_cache()
@@ -321,18 +373,18 @@ def main():
         act = torch.empty((Pm, Im), dtype=torch.bfloat16, device=dev)
         aq = torch.empty((Pm, Im), dtype=torch.float8_e4m3fn, device=dev)
         asc = torch.empty((Pm, Im // 128), dtype=torch.float32, device=dev)
-        us = _time_calls(lambda: silu_and_mul_fwd(h1, act), 30, 5)
+        us = _time_calls(lambda: silu_and_mul_fwd(h1, act), 10, 5)
         byts = Pm * Im * 6
         others.append({"name": f"silu_and_mul [{Pm},{2 * Im}]", "us": round(us, 2), "GB/s": round(byts / us / 1e3, 1),
                        "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
-        us = _time_calls(lambda: silu_and_mul_post_quant_fwd(h1, aq, asc), 30, 5)
+        us = _time_calls(lambda: silu_and_mul_post_quant_fwd(h1, aq, asc), 10, 5)
         byts = Pm * Im * 5 + Pm * (Im // 128) * 4
         others.append({"name": f"silu_and_mul + group quant fused [{Pm},{2 * Im}]", "us": round(us, 2),
                        "GB/s": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
         del h1, act, aq, asc
         h3 = make_act(Pm, Hm, 51, dev).view(Pm // topk_m, topk_m, Hm)
         red = torch.empty((Pm // topk_m, Hm), dtype=torch.bfloat16, device=dev)
-        us = _time_calls(lambda: moe_sum_reduce(h3, red), 30, 5)
+        us = _time_calls(lambda: moe_sum_reduce(h3, red), 10, 5)
         byts = (Pm + Pm // topk_m) * Hm * 2
         others.append({"name": f"moe_sum_reduce [{Pm // topk_m},{topk_m},{Hm}]", "us": round(us, 2),
                        "GB/s": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
@@ -343,7 +395,7 @@ def main():
         # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
-        us = _time_calls(lambda: dst.copy_(src), 5, 2)
+        us = _time_calls(lambda: dst.copy_(src), 5, 2, batches=3)
         others.append({"name": "copy 1 GiB (reads 2^30 B, writes 2^30 B per launch)", "us": round(us, 1),
                        "GB/s": round(2 * (1 << 30) / us / 1e3, 1)})
 

@@ -110,6 +110,9 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
 #define MI355_GEMM_TILE256x128 5 /* 256x128x128 CTA tile, 8 waves */
 #define MI355_GEMM_TILE256_RING 6 /* the 256x256 tile on the plain ring pipeline (comparison / any scale layout) */
 #define MI355_GEMM_TILE256_ONCE 7 /* MI355_GEMM_TILE256 with one workgroup per tile even when a workspace is given */
+#define MI355_GEMM_TILE256_STREAMK 8 /* the 256x256 tile with the K steps of all tiles shared evenly between the
+                                        compute units (partial tiles added up through the workspace, in K order:
+                                        deterministic); falls back to MI355_GEMM_TILE256 where sharing gains nothing */
 
 #define MI355_WS_COUNTER_BYTES 65536
 

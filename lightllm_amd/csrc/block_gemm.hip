@@ -68,26 +68,70 @@ static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false>(a, grid, st);
 }
 
+// Stream-K plan of the 256x256 kernel: the number of workgroups (one per compute unit, a multiple of 8), or 0 when
+// the tiles fill whole rounds anyway or there is too little work to give every unit 16 K steps (the 128x128
+// split-K tiles take those shapes).
+static int stream_k_groups(int64_t tiles, int64_t KB, int cus) {
+    if (cus < 8 || tiles <= 0 || tiles > 16384 - PPCfg::kTileCounterWord) return 0;
+    const int64_t units = tiles * KB;
+    if (units >= (1ll << 31)) return 0;
+    const int64_t groups = cus / 8 * 8;
+    if (units / 16 < groups || tiles % groups == 0) return 0;
+    return (int)groups;
+}
+
+// Whether the shape table should take that plan.  A workgroup that shares tiles no longer runs in step with the
+// ones that read the same X and W panels, so its K steps are served by the memory side instead of the L2 and take
+// about 2.5 times as long: sharing pays only where the plain loop leaves most of the device idle.
+static bool stream_k_pays(int64_t tiles, int64_t KB, int cus) {
+    const int groups = stream_k_groups(tiles, KB, cus);
+    if (groups == 0) return false;
+    const int64_t plain = (tiles + groups - 1) / groups * KB, shared = (tiles * KB + groups - 1) / groups;
+    return shared * 5 <= plain * 2;
+}
+
+static size_t stream_k_workspace(int groups) {
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)2 * groups * PPCfg::kPartialBytes;
+}
+
 // The 256x256 ping-pong kernel.  a.tiles_m / a.tiles_n / a.total_tiles are set by the caller.  With a workspace
 // whose counter words are zero the launch is persistent (one workgroup per CU, tiles handed out per XCD);
-// without one every workgroup runs a single tile.  Returns MI355_EUNSUPPORTED when the K range does not fit
-// the kernel's LDS layout or the X scales cannot be fetched in chunks.
+// without one every workgroup runs a single tile.  `sk_groups` > 0 asks for the stream-K launch with that many
+// workgroups (dense only; the workspace must hold stream_k_workspace(sk_groups)).  Returns MI355_EUNSUPPORTED
+// when the K range does not fit the kernel's LDS layout.
+template <bool GROUPED, bool SK, bool SC4>
+static int launch_pp_as(GemmArgs &a, int grid, int lds_bytes, hipStream_t st) {
+    constexpr auto kernel = block_fp8_gemm_pp_kernel<GROUPED, SK, SC4>;
+    if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
+    return launch(kernel, dim3(grid), dim3(PPCfg::kThreads), lds_bytes, st, a);
+}
+
 template <bool GROUPED>
-static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hipStream_t st) {
-    if (!chunked_scales_ok(a)) return MI355_EUNSUPPORTED;
+static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, int sk_groups, hipStream_t st) {
     const int lds_bytes = PPCfg::lds_bytes(a.K / kBlockK);
     if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
-    constexpr auto kernel = block_fp8_gemm_pp_kernel<GROUPED>;
-    if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
+    if (a.xs_m < 0 || a.xs_k < 0) return MI355_EUNSUPPORTED;
+    const bool sc4 = chunked_scales_ok(a);
     a.blocks_per_xcd = (a.total_tiles + 7) / 8;
     int per_xcd = a.blocks_per_xcd;
     a.counters = nullptr;
+    const bool ws_ok = ws && ((uintptr_t)ws & 15) == 0;
+    if constexpr (!GROUPED) {
+        if (sk_groups > 0) {
+            if (!ws_ok || ws_bytes < stream_k_workspace(sk_groups)) return MI355_EWORKSPACE;
+            a.counters = (uint32_t *)ws;
+            a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+            return sc4 ? launch_pp_as<false, true, true>(a, sk_groups, lds_bytes, st)
+                       : launch_pp_as<false, true, false>(a, sk_groups, lds_bytes, st);
+        }
+    }
     // persistent only when there is more than one tile per CU (a single round gains nothing from the tile queue)
-    if (ws && ws_bytes >= (size_t)MI355_WS_COUNTER_BYTES && ((uintptr_t)ws & 3) == 0 && per_xcd > cus / 8 && cus >= 8) {
+    if (ws_ok && ws_bytes >= (size_t)MI355_WS_COUNTER_BYTES && per_xcd > cus / 8 && cus >= 8) {
         a.counters = (uint32_t *)ws;
         per_xcd = cus / 8;
     }
-    return launch(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_bytes, st, a);
+    return sc4 ? launch_pp_as<GROUPED, false, true>(a, per_xcd * 8, lds_bytes, st)
+               : launch_pp_as<GROUPED, false, false>(a, per_xcd * 8, lds_bytes, st);
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE = kDense>
@@ -180,10 +224,19 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
            ((uintptr_t)B & 15) == 0;
 }
 
-static int pick_variant(int64_t M, int64_t N, int cus) {
+// The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
+//   M <= 64                                          weight streaming
+//   few 256x256 tiles, long K                        stream-K (the plain loop would leave most units idle)
+//   128x128 tiles fit one round of two per unit and
+//     (few 256x256 tiles or a short K)               128x128 tiles, K shared between workgroups when they are few
+//   otherwise                                        256x256 ping-pong tiles
+static int pick_variant(int64_t M, int64_t N, int64_t K, int cus) {
     if (M <= 64) return MI355_GEMM_SKINNY;
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    // measured crossover (N=7168, K=18432): 56 tiles of 256x256 lose to split-K 128x128 tiles, 112 tiles win
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+    const int64_t KB = K / kBlockK;
+    if (M > 128 && stream_k_pays(t256, KB, cus)) return MI355_GEMM_TILE256_STREAMK;
+    if (t128 <= 2 * (int64_t)cus && (t256 < (int64_t)cus * 3 / 8 || KB <= 64)) return MI355_GEMM_TILE128;
     if (t256 >= (int64_t)cus * 3 / 8) return MI355_GEMM_TILE256;
     return MI355_GEMM_TILE128;
 }
@@ -213,7 +266,11 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     if (K % kBlockK != 0) return 0;
     // sized from the launch plan of the current device (256 compute units when no device is visible)
     const int cus = device_cus();
-    if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, cus);
+    if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, K, cus);
+    if (variant == MI355_GEMM_TILE256_STREAMK) {
+        const int groups = stream_k_groups(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus);
+        return groups > 0 ? stream_k_workspace(groups) : (size_t)MI355_WS_COUNTER_BYTES;
+    }
     if (variant == MI355_GEMM_TILE128) {
         const int splits = tile128_splits(M, N, K, cus);
         return splits > 1 ? tile128_workspace(M, N, splits) : 0;
@@ -244,7 +301,11 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
                       256 * lda < (1ll << 32) && 256 * ldb_n < (1ll << 32) && 256 * as_m * 4 < (1ll << 32) &&
                       as_m >= 0 && as_k >= 0;
     if (variant == MI355_GEMM_AUTO) {
-        variant = fast ? pick_variant(M, N, cus) : MI355_GEMM_GENERIC;
+        variant = fast ? pick_variant(M, N, K, cus) : MI355_GEMM_GENERIC;
+        // stream-K needs its partial-tile slots; without them the plain tile loop gives the same result
+        if (variant == MI355_GEMM_TILE256_STREAMK &&
+            (!ws || ws_bytes < mi355_block_fp8_gemm_workspace_bytes(M, N, K, variant) || ((uintptr_t)ws & 15)))
+            variant = MI355_GEMM_TILE256;
         // the stream kernel's own limits are not errors under AUTO: the 128x128 tile takes every fast layout
         // and runs unsplit without a workspace
         if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
@@ -282,15 +343,17 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
         case MI355_GEMM_TILE256_ONCE:  // kept for comparison
             ws = nullptr;
             [[fallthrough]];
-        case MI355_GEMM_TILE256: {
-            // the ping-pong kernel fetches X scales eight K steps at a time (row-major scales, 16-byte aligned
-            // rows); other layouts take the plain ring
+        case MI355_GEMM_TILE256:
+        case MI355_GEMM_TILE256_STREAMK: {
             a.tiles_m = (a.M + 255) / 256;
             a.tiles_n = (a.N + 255) / 256;
             a.total_tiles = a.tiles_m * a.tiles_n;
-            const int r = launch_pp<false>(a, ws, ws_bytes, cus, st);
+            // stream-K when asked for and worth it on this device; the plain tile loop otherwise
+            const int groups =
+                variant == MI355_GEMM_TILE256_STREAMK ? stream_k_groups(a.total_tiles, a.K / kBlockK, cus) : 0;
+            const int r = launch_pp<false>(a, ws, ws_bytes, cus, groups, st);
             if (r != MI355_EUNSUPPORTED) return r;
-            return launch_dense<256, 256, 2, 4, 2>(a, st);
+            return launch_dense<256, 256, 2, 4, 2>(a, st);  // K ranges past the ping-pong kernel's LDS layout
         }
         case MI355_GEMM_TILE256_RING:  // kept for comparison
             return launch_dense<256, 256, 2, 4, 2>(a, st);
@@ -458,7 +521,7 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
         case 128: return launch_tile<128, 128, 2, 2, 2, kGrouped>(a, finish(128), st);
         case 256:
             finish(256);
-            return launch_pp<true>(a, ws, ws_bytes, device_cus(), st);
+            return launch_pp<true>(a, ws, ws_bytes, device_cus(), 0, st);
         default: return MI355_EINVAL;
     }
 }

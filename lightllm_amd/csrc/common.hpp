@@ -74,6 +74,22 @@ __device__ __forceinline__ void dma_g2l_b32(uint32_t lds_base, const void *gbase
         : "memory");
 }
 
+// 16-byte loads and stores that read past / write through the per-XCD L2 (cache policy sc1, what an agent-scope
+// relaxed atomic access compiles to on gfx950), for data exchanged between workgroups of one launch.  They are
+// ordinary memory operations to the compiler, so a batch of loads is issued back to back and waited for once.
+// The buffer resource covers 2 GiB from `base`.
+struct Sc1Buffer {
+    __amdgpu_buffer_rsrc_t rsrc;
+    __device__ __forceinline__ explicit Sc1Buffer(const void *base)
+        : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x7fffffff, 0x00020000)) {}
+    __device__ __forceinline__ v4f load(uint32_t byte_off) const {
+        return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_off, 0, 16));
+    }
+    __device__ __forceinline__ void store(uint32_t byte_off, v4f v) const {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), rsrc, (int)byte_off, 0, 16);
+    }
+};
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     // gfx9 encoding of s_waitcnt: vmcnt low bits [3:0], high bits [15:14]; expcnt [6:4]=7, lgkmcnt [11:8]=15 (no wait).

@@ -29,6 +29,17 @@
 //     per XCD in the caller's workspace, fetched two tiles ahead; the schedule-table row of a tile is loaded one
 //     tile ahead.  Counter words: [0..7] per-XCD, [8] workgroups that have finished; the last one to finish
 //     zeroes them again.  Without a workspace (counters == nullptr) every workgroup runs one tile.
+//   * Stream-K launch (SK, dense only): when the tiles do not fill whole rounds of the device, the K steps of all
+//     tiles - tile-major, in the dense tile order - are cut into one contiguous run per workgroup, so every compute
+//     unit does the same number of K steps.  A workgroup whose run covers only part of a tile's K range writes its
+//     fp32 accumulators to its own slot of the workspace (two slots per workgroup: a run starts and ends inside at
+//     most one tile each) and bumps the tile's arrival counter; whoever arrives last adds the tile's partials in K
+//     order (so the result does not depend on who that is), stores the tile and re-zeroes the counter.  Nobody
+//     waits for anybody.
+//   * SC4: the X scales are row-major with 16-byte aligned rows and K/128 a multiple of 8, and a chunk is fetched
+//     with one 16-byte request per half row.  Otherwise (any strides, any K/128) it is fetched with 4-byte
+//     requests, one per (row, step), four instructions per wave and chunk; steps past the end of K repeat the
+//     last one.
 #pragma once
 #include "gemm_tile.hpp"
 
@@ -48,10 +59,13 @@ struct PPCfg {
     static constexpr int sched_off(int KB) { return chunk_off(KB) + 2 * kChunkBytes; }
     static constexpr int lds_bytes(int KB) { return sched_off(KB) + 16; }
     static constexpr int kCounterWords = 9;
+    static constexpr int kTileCounterWord = 16;       // stream-K: arrival counters of the tiles start here
+    static constexpr int kPartialBytes = BM * BN * 4;  // one fp32 partial tile
 };
 
-template <bool GROUPED>
+template <bool GROUPED, bool SK, bool SC4>
 __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p) {
+    static_assert(!(GROUPED && SK), "stream-K is a dense launch");
     using Cfg = PPCfg;
     constexpr int BM = Cfg::BM, TM = Cfg::TM, TN = Cfg::TN, HM = Cfg::HM, WMS = Cfg::WMS, WNS = Cfg::WNS;
     constexpr bool SKIP = GROUPED;  // ragged tiles skip empty halves; dense tiles keep the branch-free body
@@ -64,10 +78,15 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     const int r16 = lane & 15, g4 = lane >> 4;
     const int sub = lane >> 3;
     const uint32_t pch = (uint32_t)(lane & 7);
-    const int KB = p.K / kBlockK, nk = KB, nchunk = KB >> 3;
+    const int KB = p.K / kBlockK, nchunk = (KB + 7) >> 3;
     const uint32_t lds0 = lds_addr(lds);
     const uint32_t xcd = blockIdx.x & 7u, in_xcd = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
-    const bool persistent = p.counters != nullptr;
+    const bool persistent = !SK && p.counters != nullptr;
+    // stream-K: this workgroup's run of (tile, K step) units; workgroups are ranked XCD-major so that one XCD works
+    // on neighbouring tiles
+    const uint32_t rank = xcd * per_xcd + in_xcd;
+    const uint64_t units = (uint64_t)p.total_tiles * (uint64_t)KB;
+    const uint32_t u_end = SK ? (uint32_t)(((uint64_t)rank + 1u) * units / gridDim.x) : 0u;
     volatile uint32_t *sched = (volatile uint32_t *)(lds + Cfg::sched_off(KB));
     constexpr uint32_t kNone = 0xffffffffu;
 
@@ -92,7 +111,19 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         int n0;
         int rows;    // valid rows
         int expert;
+        int k0, k1;  // K steps [k0, k1) of the tile that this workgroup computes (the whole range unless SK)
+        uint32_t id; // stream-K: logical tile number
         bool valid;
+    };
+    auto dense_coords = [&](uint32_t logical, uint32_t &tile_m, uint32_t &tile_n) {
+        constexpr uint32_t GM = 8;
+        const uint32_t width = GM * (uint32_t)p.tiles_n;
+        const uint32_t g = logical / width;
+        const uint32_t first_m = g * GM;
+        const uint32_t gsz = min((uint32_t)p.tiles_m - first_m, GM);
+        const uint32_t in_grp = logical - g * width;
+        tile_m = first_m + in_grp % gsz;
+        tile_n = in_grp / gsz;
     };
     auto tile_coords = [&](uint32_t v, uint32_t &tile_m, uint32_t &tile_n) -> bool {
         if (v == kNone) return false;
@@ -105,14 +136,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
             if (v >= (uint32_t)p.blocks_per_xcd) return false;
             const uint32_t logical = xcd * (uint32_t)p.blocks_per_xcd + v;
             if (logical >= (uint32_t)p.total_tiles) return false;
-            constexpr uint32_t GM = 8;
-            const uint32_t width = GM * (uint32_t)p.tiles_n;
-            const uint32_t g = logical / width;
-            const uint32_t first_m = g * GM;
-            const uint32_t gsz = min((uint32_t)p.tiles_m - first_m, GM);
-            const uint32_t in_grp = logical - g * width;
-            tile_m = first_m + in_grp % gsz;
-            tile_n = in_grp / gsz;
+            dense_coords(logical, tile_m, tile_n);
         }
         return true;
     };
@@ -122,10 +146,21 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         if (!GROUPED || !tile_coords(v, tm, tn)) return v4i{-1, 0, 0, 0};
         return *(const v4i *)(p.table + (int64_t)tm * 4);
     };
+    // non-SK: v is a sequence number; SK: v is the first unit of the segment
     auto make_tile = [&](uint32_t v, v4i row) -> Tile {
-        Tile t = {0, 0, 0, 0, false};
+        Tile t = {0, 0, 0, 0, 0, KB, 0u, false};
         uint32_t tm = 0, tn = 0;
-        if (!tile_coords(v, tm, tn)) return t;
+        if constexpr (SK) {
+            if (v >= u_end) return t;
+            t.id = v / (uint32_t)KB;
+            t.k0 = (int)(v - t.id * (uint32_t)KB);
+            t.k1 = min(KB, t.k0 + (int)(u_end - v));
+            t.k0 = __builtin_amdgcn_readfirstlane(t.k0);
+            t.k1 = __builtin_amdgcn_readfirstlane(t.k1);
+            dense_coords(t.id, tm, tn);
+        } else {
+            if (!tile_coords(v, tm, tn)) return t;
+        }
         t.n0 = (int)tn * Cfg::BN;
         if constexpr (GROUPED) {
             t.expert = __builtin_amdgcn_readfirstlane(row[0]);
@@ -145,6 +180,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
 
     // ---- per-tile request state
     uint32_t xoff[Cfg::XI], woff[Cfg::WI], sc_off = 0;
+    uint32_t sc_row[SC4 ? 1 : Cfg::XI];  // !SC4: scale-row offsets (elements) of the rows this lane fetches
     bool x_real[Cfg::XI];
     bool do_half0 = true, do_half1 = true;
     const uint8_t *xg = p.X, *wg = p.W;
@@ -191,6 +227,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
             const uint32_t src_row = GROUPED ? raw[i] / (uint32_t)p.topk : raw[i];
             xoff[i] = src_row * (uint32_t)p.ldx + c * 16u;
             x_real[i] = !SKIP || (wave + i * Cfg::kWaves) * 8 < t.rows;
+            if constexpr (!SC4) sc_row[i] = src_row * (uint32_t)p.xs_m;
         }
         const uint32_t srow = GROUPED ? raw[Cfg::XI] / (uint32_t)p.topk : raw[Cfg::XI];
         sc_off = (srow * (uint32_t)p.xs_m + 4u * (uint32_t)(lane & 1)) * 4u;
@@ -237,10 +274,20 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
 #pragma unroll
         for (int i = 1; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
     };
-    // lane l of wave w fetches steps 4*(l&1).. of row 32*w + l/2 of the chunk: scale (row, kb) then sits at
-    // chunk[(kb/8) & 1][row][kb % 8]
+    // Scale (row, kb) sits at chunk[(kb/8) & 1][row][kb % 8].  SC4: lane l of wave w fetches steps 4*(l&1).. of row
+    // 32*w + l/2.  Otherwise lane l fetches step l%8 of row l/8 of the same four 8-row groups it fetches X rows
+    // for; steps past the end of K repeat the last step (never read).
     auto issue_scales = [&](int chunk) {
-        dma_g2l_b128(lds0 + chunk_off + (uint32_t)(chunk & 1) * Cfg::kChunkBytes + (uint32_t)wave * 1024u, sg + 8 * chunk, sc_off);
+        const uint32_t dst = lds0 + chunk_off + (uint32_t)(chunk & 1) * Cfg::kChunkBytes;
+        if constexpr (SC4) {
+            dma_g2l_b128(dst + (uint32_t)wave * 1024u, sg + 8 * chunk, sc_off);
+        } else {
+            const uint32_t st = (uint32_t)min(lane & 7, KB - 1 - 8 * chunk) * (uint32_t)p.xs_k;
+            const float *sk = sg + (int64_t)(8 * chunk) * p.xs_k;
+#pragma unroll
+            for (int i = 0; i < Cfg::XI; ++i)
+                dma_g2l_b32(dst + (uint32_t)(wave + i * Cfg::kWaves) * 256u, sk, (sc_row[i] + st) * 4u);
+        }
     };
     constexpr int kXhi = Cfg::XI / 2;             // requests per wave in A0
     constexpr int kWXlo = Cfg::XI / 2 + Cfg::WI;  // requests per wave in A1
@@ -258,21 +305,29 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     uint32_t v_next = persistent ? per_xcd + in_xcd : kNone;  // sequence number of the tile after the current one
     uint32_t v_after = kNone;                                 // and of the one after that (fetched)
     uint32_t fetched = 0;
-    Tile cur = make_tile(in_xcd, load_row(in_xcd));
+    const uint32_t v_first = SK ? (uint32_t)((uint64_t)rank * units / gridDim.x) : in_xcd;
+    Tile cur = make_tile(v_first, load_row(in_xcd));
     v4i row_next = load_row(v_next);
     if (persistent && tid == 0)
         fetched = __hip_atomic_fetch_add(p.counters + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // the first requests of a tile: both W slots, the scale chunk(s) of the first steps, X of the first step and
+    // the first half of the second
+    auto first_requests = [&](const Tile &t, const uint32_t (&raw)[Cfg::XI + 1]) {
+        const int k1 = t.k0 + min(1, t.k1 - t.k0 - 1);  // second step (the first again for a one-step range)
+        setup_w(t);
+        issue_w(0, t.k0);
+        issue_w(1, k1);
+        setup_x(t, raw);
+        issue_scales(t.k0 >> 3);
+        if (SK && (t.k0 & 7) != 0 && (t.k0 >> 3) + 1 < nchunk) issue_scales((t.k0 >> 3) + 1);
+        issue_xlo(0, t.k0);
+        issue_xhi(0, t.k0);
+        issue_xlo(1, k1);
+    };
     if (cur.valid) {
         uint32_t raw[Cfg::XI + 1];
         gather(cur, raw);
-        setup_w(cur);
-        issue_w(0, 0);
-        issue_w(1, min(1, nk - 1));
-        setup_x(cur, raw);
-        issue_scales(0);
-        issue_xlo(0, 0);
-        issue_xhi(0, 0);
-        issue_xlo(1, min(1, nk - 1));
+        first_requests(cur, raw);
         ws_store(cur, 0, ws_load(cur));
     }
     wait_vmcnt<0>();
@@ -280,6 +335,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     __syncthreads();
     if (persistent) v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
 
+    uint32_t u_pos = v_first;  // stream-K: first unit of the current segment
     v4f acc[TM][TN];
     while (cur.valid) {
 #pragma unroll
@@ -291,12 +347,13 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         // ---- the K loop
         if (grp == 1) phase_end();
         int slot = 0;
-        for (int it = 0; it < nk; ++it) {
+        const int kfirst = cur.k0, klast = cur.k1 - 1;
+        for (int kb = kfirst; kb <= klast; ++kb) {
             const uint8_t *st = lds + slot * Cfg::kStage;
-            const int cbuf = (it >> 3) & 1;
+            const int cbuf = (kb >> 3) & 1;
             // A0 (LDS reads first: a DMA request can stall the wave's issue, the reads behind it would wait)
-            const float ws_cur = wsl[it];
-            const float *sp = (const float *)(lds + sr8 + cbuf * Cfg::kChunkBytes + (it & 7) * 4);
+            const float ws_cur = wsl[kb];
+            const float *sp = (const float *)(lds + sr8 + cbuf * Cfg::kChunkBytes + (kb & 7) * 4);
             v8i wf[TN], xf[HM];
             if (do_half0) {
 #pragma unroll
@@ -320,11 +377,11 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
                     }
                 }
                 if (h == 0) {
-                    if ((it & 7) == 0 && (it >> 3) + 1 < nchunk) issue_scales((it >> 3) + 1);
-                    issue_xhi(slot ^ 1, min(it + 1, nk - 1));
+                    if ((kb & 7) == 0 && (kb >> 3) + 1 < nchunk) issue_scales((kb >> 3) + 1);
+                    issue_xhi(slot ^ 1, min(kb + 1, klast));
                 } else {
-                    issue_xlo(slot, min(it + 2, nk - 1));
-                    issue_w(slot, min(it + 2, nk - 1));
+                    issue_xlo(slot, min(kb + 2, klast));
+                    issue_w(slot, min(kb + 2, klast));
                 }
                 // everything but the last two request groups has landed: at the end of A0 that covers the second
                 // X half of this step, at the end of A1 the W rows and first X half of the next one (the scale
@@ -362,13 +419,16 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         // ---- between two tiles: first requests of the next tile, then the stores of this one
         const Tile done = cur;
         float ws_first = 0.f;
-        cur = make_tile(v_next, row_next);
+        if constexpr (SK) {
+            u_pos += (uint32_t)(done.k1 - done.k0);
+            cur = make_tile(u_pos, v4i{-1, 0, 0, 0});
+        } else {
+            cur = make_tile(v_next, row_next);
+        }
         if (cur.valid) {
             uint32_t raw[Cfg::XI + 1];
             gather(cur, raw);
-            setup_w(cur);
-            issue_w(0, 0);
-            issue_w(1, min(1, nk - 1));
+            first_requests(cur, raw);
             // sequence number and table row for later tiles (used one and two tiles from now)
             v_next = v_after;
             row_next = load_row(v_next);
@@ -376,16 +436,63 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
                 fetched = __hip_atomic_fetch_add(p.counters + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             wsbuf ^= 1;
             ws_first = ws_load(cur);
-            setup_x(cur, raw);
-            issue_scales(0);
-            issue_xlo(0, 0);
-            issue_xhi(0, 0);
-            issue_xlo(1, min(1, nk - 1));
+        }
+
+        // ---- stream-K: a part of a tile goes to the workspace; the last part to arrive adds them all up
+        bool store_tile = true;
+        if constexpr (SK) {
+            if (done.k0 != 0 || done.k1 != KB) {  // the same for the whole workgroup
+                constexpr uint32_t kBlockStride = Cfg::kThreads * 16;  // bytes between a lane's 16x16 blocks
+                const Sc1Buffer xch(p.partials);
+                const uint32_t lane_off = (uint32_t)tid * 16u;
+                const uint32_t mine = (2u * rank + (done.k0 == 0 ? 1u : 0u)) * (uint32_t)Cfg::kPartialBytes + lane_off;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) xch.store(mine + (uint32_t)(i * TN + j) * kBlockStride, acc[i][j]);
+                wait_vmcnt<0>();
+                __syncthreads();
+                // the ranks that hold parts of this tile: those whose runs contain its first and its last unit
+                const uint64_t t0 = (uint64_t)done.id * (uint64_t)KB;
+                const uint32_t r_lo = (uint32_t)(((t0 + 1u) * gridDim.x - 1u) / units);
+                const uint32_t r_hi = (uint32_t)(((t0 + (uint64_t)KB) * gridDim.x - 1u) / units);
+                uint32_t *counter = p.counters + Cfg::kTileCounterWord + done.id;
+                if (tid == 0) sched[0] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                store_tile = sched[0] == r_hi - r_lo;
+                if (store_tile) {
+                    // parts in K order: the first rank's run ends inside the tile (its second slot), every later
+                    // one starts inside it (its first slot).  The first part is loaded straight into the
+                    // accumulators, the others in halves.
+                    const uint32_t first = (2u * r_lo + 1u) * (uint32_t)Cfg::kPartialBytes + lane_off;
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) acc[i][j] = xch.load(first + (uint32_t)(i * TN + j) * kBlockStride);
+                    for (uint32_t r = r_lo + 1; r <= r_hi; ++r) {
+                        const uint32_t src = 2u * r * (uint32_t)Cfg::kPartialBytes + lane_off;
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            v4f part[TM / 2][TN];
+#pragma unroll
+                            for (int i = 0; i < TM / 2; ++i)
+#pragma unroll
+                                for (int j = 0; j < TN; ++j)
+                                    part[i][j] = xch.load(src + (uint32_t)((h * (TM / 2) + i) * TN + j) * kBlockStride);
+#pragma unroll
+                            for (int i = 0; i < TM / 2; ++i)
+#pragma unroll
+                                for (int j = 0; j < TN; ++j) acc[h * (TM / 2) + i][j] += part[i][j];
+                        }
+                    }
+                    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
         }
 
         // epilogue of the finished tile: lane (r16, g4) holds, for each tm, row wave_m*WMS + 16*tm + r16 and, for
         // each block pair h, the 8 columns n0 + wave_n*WNS + lane_col(g4, 2h) + [0, 8)
-        {
+        if (store_tile) {
             const int nbase = done.n0 + wave_n * WNS;
             const int32_t *idx_list = GROUPED ? p.e2t_index + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
             const float *w_list = GROUPED ? p.e2t_weight + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;

@@ -249,16 +249,13 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
     }
 
     if constexpr (SPLIT) {
-        // same exchange protocol as the tiled split-K kernel: agent-scope relaxed atomics, no cache-wide fence
-        float *mine = p.partials + ((int64_t)tile_n * p.splits + split) * Cfg::kTileElems;
+        // same exchange protocol as the tiled split-K kernel (sc1 stores and loads, no cache-wide fence)
+        const Sc1Buffer xch(p.partials + (int64_t)tile_n * p.splits * Cfg::kTileElems);
+        const uint32_t lane_off = (uint32_t)lane * 16u;
 #pragma unroll
         for (int q = 0; q < FW; ++q) {
             const int f = q * kStreamWaves + wave;
-            if (f < F) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    __hip_atomic_store(mine + (f * 64 + lane) * 4 + v, sum[q][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            if (f < F) xch.store(split * (uint32_t)(Cfg::kTileElems * 4) + (uint32_t)f * 1024u + lane_off, sum[q]);
         }
         wait_vmcnt<0>();
         __syncthreads();
@@ -267,19 +264,25 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
             *arrived = __hip_atomic_fetch_add(p.counters + tile_n, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*arrived != (uint32_t)p.splits - 1u) return;
-        const float *base = p.partials + (int64_t)tile_n * p.splits * Cfg::kTileElems;
+        // the last workgroup adds the partials in split order, four splits per memory round trip
+        constexpr int kBatch = 4;
+        for (int sp0 = 0; sp0 < p.splits; sp0 += kBatch) {
+            v4f t[FW][kBatch];
 #pragma unroll
-        for (int q = 0; q < FW; ++q) {
-            const int f = q * kStreamWaves + wave;
-            v4f s = v4f{0.f, 0.f, 0.f, 0.f};
-            if (f < F) {
-                for (int sp = 0; sp < p.splits; ++sp) {
-                    const float *src = base + (int64_t)sp * Cfg::kTileElems + (f * 64 + lane) * 4;
+            for (int q = 0; q < FW; ++q) {
+                const int f = q * kStreamWaves + wave;
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) s[v] += __hip_atomic_load(src + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+                for (int d = 0; d < kBatch; ++d)
+                    if (f < F && sp0 + d < p.splits)
+                        t[q][d] = xch.load((uint32_t)(sp0 + d) * (uint32_t)(Cfg::kTileElems * 4) + (uint32_t)f * 1024u + lane_off);
             }
-            sum[q] = s;
+#pragma unroll
+            for (int q = 0; q < FW; ++q) {
+                const int f = q * kStreamWaves + wave;
+#pragma unroll
+                for (int d = 0; d < kBatch; ++d)
+                    if (f < F && sp0 + d < p.splits) sum[q] = (sp0 + d == 0) ? t[q][d] : sum[q] + t[q][d];
+            }
         }
         if (tid == 0) __hip_atomic_store(p.counters + tile_n, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }

@@ -364,22 +364,26 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
 
 
     // ---- split-K: publish the partial, let the last CTA of the tile reduce
-    // Partials and the arrival counter are exchanged with agent-scope relaxed atomics: such stores write
-    // through, and such loads read past, the per-XCD L2, so no cache-wide write-back / invalidate fence is
-    // needed (one of those per CTA costs more than the whole GEMM at decode sizes).  Order is kept by
+    // Partials are exchanged with sc1 accesses and the arrival counter with an agent-scope relaxed atomic: such
+    // stores write through, and such loads read past, the per-XCD L2, so no cache-wide write-back / invalidate
+    // fence is needed (one of those per CTA costs more than the whole GEMM at decode sizes).  Order is kept by
     // "all my stores acknowledged (vmcnt 0) -> barrier -> one atomic add" on the writer side and
-    // "atomic add returned -> barrier -> loads" on the reader side.
+    // "atomic add returned -> barrier -> loads" on the reader side.  What this relies on: a gfx950 store with
+    // sc1 is complete (vmcnt) only once it has reached the memory side that all XCDs share, and a load with sc1
+    // is served from there, never from a line the reader's own L2 or L1 held before.
     if constexpr (MODE == kSplitK) {
         constexpr int kTileElems = BM * BN;
-        float *mine = p.partials + ((int64_t)tile_id * p.splits + split) * kTileElems;
+        constexpr int NB = TM * TN;  // 16x16 blocks per lane, 16 bytes each
+        const float *tile_base = p.partials + (int64_t)tile_id * p.splits * kTileElems;
+        const Sc1Buffer xch(tile_base);
+        const uint32_t lane_off = (uint32_t)tid * 16u;
+        {
+            const uint32_t mine = split * (uint32_t)(kTileElems * 4) + lane_off;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    __hip_atomic_store(mine + ((i * TN + j) * Cfg::kThreads + tid) * 4 + v, acc[i][j][v], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+                for (int j = 0; j < TN; ++j) xch.store(mine + (uint32_t)((i * TN + j) * Cfg::kThreads * 16), acc[i][j]);
+        }
         wait_vmcnt<0>();
         __syncthreads();
         // (the arrival word lives in the dynamic allocation: a static __shared__ object would push static +
@@ -389,19 +393,27 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             *arrived = __hip_atomic_fetch_add(p.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*arrived != (uint32_t)p.splits - 1u) return;
-        const float *base = p.partials + (int64_t)tile_id * p.splits * kTileElems;
+        // the last workgroup adds the partials in split order; the loads of one split are in flight while the
+        // previous one is added (one memory round trip per split, not one per 16 bytes)
+        auto fetch = [&](v4f (&dst)[NB], int sp) {
+            const uint32_t src = (uint32_t)sp * (uint32_t)(kTileElems * 4) + lane_off;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int b = 0; b < NB; ++b) dst[b] = xch.load(src + (uint32_t)(b * Cfg::kThreads * 16));
+        };
+        auto add = [&](const v4f (&src)[NB], bool first) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                v4f s = v4f{0.f, 0.f, 0.f, 0.f};
-                for (int sp = 0; sp < p.splits; ++sp) {
-                    const float *q = base + (int64_t)sp * kTileElems + ((i * TN + j) * Cfg::kThreads + tid) * 4;
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) s[v] += __hip_atomic_load(q + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-                acc[i][j] = s;
-            }
+                for (int j = 0; j < TN; ++j) acc[i][j] = first ? src[i * TN + j] : acc[i][j] + src[i * TN + j];
+        };
+        v4f even[NB], odd[NB];
+        fetch(even, 0);
+        for (int sp = 0; sp < p.splits; sp += 2) {
+            if (sp + 1 < p.splits) fetch(odd, sp + 1);
+            add(even, sp == 0);
+            if (sp + 2 < p.splits) fetch(even, sp + 2);
+            if (sp + 1 < p.splits) add(odd, false);
+        }
         if (tid == 0) __hip_atomic_store(p.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 

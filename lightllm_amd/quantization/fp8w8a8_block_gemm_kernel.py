@@ -14,6 +14,7 @@ _VARIANTS = {
     None: _lib.GEMM_AUTO, "auto": _lib.GEMM_AUTO, "tile256": _lib.GEMM_TILE256, "tile128": _lib.GEMM_TILE128,
     "skinny": _lib.GEMM_SKINNY, "generic": _lib.GEMM_GENERIC, "tile256x128": _lib.GEMM_TILE256x128,
     "tile256ring": _lib.GEMM_TILE256_RING, "tile256once": _lib.GEMM_TILE256_ONCE,
+    "tile256streamk": _lib.GEMM_TILE256_STREAMK,
 }
 
 
@@ -36,7 +37,7 @@ def w8a8_block_fp8_matmul(
     A [M,K] e4m3fn contiguous; B [K,N] e4m3fn (LightLLM passes ``weight.t()``: strides (1,K));
     Ascale [M, K/128] fp32; Bscale [K/128, ceil(N/128)] fp32; C [M,N] bf16 contiguous.
     ``run_config`` may be ``{"variant": "auto"|"tile256"|"tile256x128"|"tile128"|"skinny"|"generic"}`` (plus the
-    comparison variants "tile256ring" and "tile256once"); the
+    comparison variants "tile256ring", "tile256once" and "tile256streamk"); the
     reference's tile dictionaries (BLOCK_M, ...) are accepted and ignored: the shape table is built in.
     """
     assert len(block_size) == 2

@@ -75,9 +75,9 @@ def test_ragged_edges(hip, M, N, K, variant):
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 1024), (257, 520, 1024), (700, 2112, 2048), (1024, 768, 3072)])
 def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
-    """K/128 % 8 == 0 with row-major scales takes the ping-pong schedule with chunked scale fetches; the plain ring
-    on the same 256x256 tile adds the same products in the same order, so the two must agree bit for bit.
-    Column-major scales (strides (1, M)) fall back to the ring inside the same variant."""
+    """The ping-pong schedule (scales fetched in chunks of eight K steps) and the plain ring on the same 256x256 tile
+    add the same products in the same order, so the two must agree bit for bit - with row-major scales (16-byte
+    requests) and with column-major scales (strides (1, M): 4-byte requests)."""
     print(f"gemm ping-pong vs ring M={M} N={N} K={K}", flush=True)
     xq, xs, wq, ws = _prep(M, N, K, seed=M + K, device="cuda")
     c_pp = _run(xq, xs, wq, ws, "tile256")
@@ -89,6 +89,66 @@ def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
     assert torch.equal(c_cm.view(torch.int16), c_ring.view(torch.int16))
     if M * N <= 300 * 600:
         _check_small(xq, xs, wq, ws, c_pp)
+
+
+@pytest.mark.parametrize("K", [128, 512, 1152, 1536, 2304, 7296])
+def test_pingpong_tile_off_grid_k(hip, K):
+    """K/128 not a multiple of 8 (the reference's own tuning list holds K = 512, 1152, 1536, 2304,
+    test/kernel/deepseekv3_fp8_block_gemm_tuning.py:230-251): the last scale chunk is partial, rows of the scale
+    matrix are not 16-byte aligned for odd K/128.  Bit-equal to the ring, persistent launch included."""
+    for (M, N) in [(300, 520), (4096, 4096)]:
+        print(f"gemm ping-pong off-grid K M={M} N={N} K={K}", flush=True)
+        xq, xs, wq, ws = _prep(M, N, K, seed=K + M, device="cuda")
+        c_pp = _run(xq, xs, wq, ws, "tile256")
+        c_ring = _run(xq, xs, wq, ws, "tile256ring")
+        assert torch.equal(c_pp.view(torch.int16), c_ring.view(torch.int16)), (M, N, K)
+        if M * N <= 300 * 600:
+            _check_small(xq, xs, wq, ws, c_pp)
+        else:
+            ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+            cos, rel = H.gemm_metrics(c_pp.float(), ref)
+            assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+
+
+# (M, N, K): tiles that do not fill whole rounds of 256 compute units, so that the stream-K plan is taken: one
+# round half empty (DeepSeek q_a+kv_a), a second round one eighth full, few tiles with a long K, ragged edges with
+# a K that is not a multiple of 1024
+STREAM_K_SHAPES = [(4096, 2112, 7168), (512, 36864, 7168), (1024, 7168, 18432), (1000, 8200, 4992), (1000, 2048, 16384)]
+
+
+@pytest.mark.parametrize("M,N,K", STREAM_K_SHAPES)
+def test_stream_k_launch(hip, M, N, K):
+    """Stream-K: the K steps of all tiles are shared evenly between the compute units and partial tiles are added
+    through the workspace in K order.  Against the torch fp32 dequant-matmul (whole matrix) and the float64 oracle
+    (sample); identical bits on repeated launches whoever arrives last; counter words zero afterwards.  The shape
+    table itself takes this launch only for the last shape (few tiles, long K)."""
+    from lightllm_amd import _lib
+
+    print(f"gemm stream-K M={M} N={N} K={K}", flush=True)
+    need = hip.mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_TILE256_STREAMK)
+    assert need > _lib.WS_COUNTER_BYTES, "the shape must take the stream-K plan on this device"
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + N)
+    first = _run(xq, xs, wq, ws, "tile256streamk").clone()
+    for _ in range(3):
+        assert torch.equal(_run(xq, xs, wq, ws, "tile256streamk").view(torch.int16), first.view(torch.int16))
+    if (M, N, K) == STREAM_K_SHAPES[-1]:
+        assert hip.mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_AUTO) == need
+        assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), first.view(torch.int16))
+    counters = _lib.workspace(xq.device, need)[: _lib.WS_COUNTER_BYTES]
+    assert not bool(counters.any())
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(first.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+    # against the plain tile loop: same products, another summation order for the tiles that were split
+    plain = _run(xq, xs, wq, ws, "tile256")
+    assert (first.float() - plain.float()).abs().max() <= 2 ** -7 * plain.float().abs().max()
+    rng = np.random.default_rng(M)
+    rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 6)])
+    cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 40)])
+    ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                          ws.cpu().numpy(), np.arange(len(rows)), cols)
+    got = first[rows][:, cols].float().cpu().double().numpy()
+    assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * np.abs(ref64).max()
 
 
 @pytest.mark.parametrize("M,N,K", [(4096, 16384, 1024), (4000, 16400, 1024), (1100, 16385, 1024)])
