@@ -114,6 +114,8 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
                                         compute units (partial tiles added up through the workspace, in K order:
                                         deterministic); falls back to MI355_GEMM_TILE256 where sharing gains nothing */
 
+#define MI355_GEMM_SKINNY_XSHARE 9 /* weight streaming, M <= 64, the activation block of a K step shared by the workgroup */
+
 #define MI355_WS_COUNTER_BYTES 65536
 
 /* Bytes of workspace the launch plan of the CURRENT device needs for this shape and variant (0 = none). */
@@ -191,8 +193,7 @@ int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32
  * W e4m3fn [E,N,K] contiguous; Ws fp32 [E, ceil(N/128), K/128] contiguous; out bf16 [num_pairs, N] contiguous.
  * num_pairs is only used as the row stride of expert_to_token_index / expert_to_weight (the number of (token, slot)
  * pairs in LightLLM's use); the masked expert-parallel layout passes a [E, T_pad] table with num_pairs = T_pad.
- * block_m must be one the library was built for: 16, 32, 64, 128, or 256 (256 needs K % 1024 == 0 and returns
- * MI355_EUNSUPPORTED otherwise); mi355_grouped_block_m() suggests one.
+ * block_m must be one the library was built for: 16, 32, 64, 128 or 256; mi355_grouped_block_m() suggests one.
  * workspace: optional, used by block_m = 256 only: MI355_WS_COUNTER_BYTES bytes that are zero before the launch
  * (the kernel leaves them zero).  With it the launch is persistent - one workgroup per compute unit takes tiles
  * from per-XCD counters and overlaps the first requests of a tile with the stores of the previous one;

@@ -3,6 +3,7 @@
 
 #include "gemm_pp.hpp"
 #include "gemm_stream.hpp"
+#include "gemm_xshare.hpp"
 #include "gemm_tile.hpp"
 
 namespace mi355 {
@@ -143,9 +144,7 @@ static int launch_dense(GemmArgs &a, hipStream_t st) {
     return launch_tile<BM, BN, WM, WN, NSTAGE, MODE>(a, a.blocks_per_xcd * 8, st);
 }
 
-// Weight-streaming launch for M <= 64: 64-row tiles (32-row ones in the case below; 16- and 128-row tiles measured
-// slower on the decode shapes), the K range split over CTAs only as far as needed to give every CU a CTA, and
-// never below 16 K steps per CTA (4 per wave).
+// Weight-streaming launches for M <= 64.
 static int skinny_mt(int64_t M) { return M <= 16 ? 1 : (M <= 32 ? 2 : 4); }
 
 struct SkinnyPlan {
@@ -154,12 +153,21 @@ struct SkinnyPlan {
 
 static SkinnyPlan skinny_plan(int64_t M, int64_t N, int64_t K, int cus) {
     SkinnyPlan pl;
-    // 32-row tiles when 64-row ones are fewer than the CUs and M > 16 (N=4096, K=14336: 17.7 / 22.5 us at M=32 / 64
-    // against 19.6 / 24.6; no difference at M <= 16, and slower when N alone fills the device)
-    pl.tnw = (M > 16 && (N + 63) / 64 < cus) ? 2 : 4;
+    pl.splits = 1;
+    if ((N + 63) / 64 >= cus) {
+        // N alone gives every compute unit a workgroup: 64-row tiles, whole K
+        pl.tnw = 4;
+        pl.tiles = (int)((N + 63) / 64);
+        return pl;
+    }
+    // Otherwise narrow tiles first, then K splits, until there are about two workgroups per compute unit (measured
+    // on N=4096, K=14336: 16-row tiles x 2 splits 13.1 us at M <= 8 against 14.1 for 64-row tiles x 4 splits;
+    // at M > 16, 32-row tiles x 4 splits 16.1 / 20.0 us at M = 32 / 64, 16-row tiles 18.3 / 25.8), never below 16 K
+    // steps per workgroup (4 per wave).
+    pl.tnw = M <= 16 ? 1 : 2;
     pl.tiles = (int)((N + 16 * pl.tnw - 1) / (16 * pl.tnw));
     const int KB = (int)(K / kBlockK);
-    pl.splits = (cus + pl.tiles - 1) / pl.tiles;
+    pl.splits = (2 * cus + pl.tiles - 1) / pl.tiles;
     const int max_splits = KB / 16 > 0 ? KB / 16 : 1;
     if (pl.splits > max_splits) pl.splits = max_splits;
     if (pl.splits < 1) pl.splits = 1;
@@ -215,8 +223,55 @@ static int launch_stream_mt(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStre
     switch (pl.tnw) {
         case 4: return launch_stream<MT, 4>(a, pl, ws, st);
         case 2: return launch_stream<MT, 2>(a, pl, ws, st);
+        case 1:
+            if constexpr (MT == 1) return launch_stream<1, 1>(a, pl, ws, st);
+            return MI355_EINVAL;
         default: return MI355_EINVAL;
     }
+}
+
+// ---- the second streaming kernel (activation block shared by the workgroup).  Measured against the first one on
+// the Llama decode shapes it wins only where the first is shortest of registers and N alone fills the device:
+// M = 33..64 with 128-row workgroup tiles (N=28672, K=4096, M=64: 29.7 us against 34.4); with 64-row tiles, few
+// tiles or smaller M its barrier per K step costs more than the shared activation block saves
+// (N=4096, K=14336: 21.5-25.2 us against 13.9-19.8).  Only that configuration is built.
+constexpr int kXshareDepth = 4;
+using XshareCfg = ShareCfg<4, 2, kXshareDepth>;
+
+static bool xshare_pays(int64_t M, int64_t N, int64_t K, int cus) {
+    return M > 32 && M <= 64 && (N + 127) / 128 >= (int64_t)cus * 3 / 4 && K / kBlockK <= XshareCfg::kMaxScaleSteps;
+}
+
+// 128-row workgroup tiles; the K range is split in two while that leaves fewer than two workgroups per compute unit
+// (224 tiles unsplit take 34.7 us on N=28672, K=4096, M=64; split in two, 29.7), never below 8 K steps each.
+static int xshare_splits(int64_t N, int64_t K, int cus) {
+    const int64_t tiles = (N + XshareCfg::BN - 1) / XshareCfg::BN, KB = K / kBlockK;
+    return tiles < 2 * (int64_t)cus && KB >= 16 ? 2 : 1;
+}
+
+static size_t xshare_workspace(int64_t N, int splits) {
+    const int64_t tiles = (N + XshareCfg::BN - 1) / XshareCfg::BN;
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * XshareCfg::kTileElems * 4;
+}
+
+static int launch_xshare(GemmArgs &a, int splits, void *ws, hipStream_t st) {
+    const int KB = a.K / kBlockK;
+    const int steps = (KB + splits - 1) / splits;
+    if (steps > XshareCfg::kMaxScaleSteps) return MI355_EUNSUPPORTED;
+    constexpr int max_lds = XshareCfg::kLds + XshareCfg::scale_lds_bytes(XshareCfg::kMaxScaleSteps);
+    const int lds_bytes = XshareCfg::kLds + XshareCfg::scale_lds_bytes(steps);
+    const int tiles = (a.N + XshareCfg::BN - 1) / XshareCfg::BN;
+    if (splits <= 1) {
+        constexpr auto kernel = block_fp8_gemm_xshare_kernel<4, 2, kXshareDepth, false>;
+        if (!allow_lds<kernel>(max_lds)) return MI355_ELAUNCH;
+        return launch(kernel, dim3(tiles), dim3(256), lds_bytes, st, a);
+    }
+    constexpr auto kernel = block_fp8_gemm_xshare_kernel<4, 2, kXshareDepth, true>;
+    if (!allow_lds<kernel>(max_lds)) return MI355_ELAUNCH;
+    a.splits = splits;
+    a.counters = (uint32_t *)ws;
+    a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+    return launch(kernel, dim3(tiles * splits), dim3(256), lds_bytes, st, a);
 }
 
 static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n) {
@@ -225,12 +280,14 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 }
 
 // The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
-//   M <= 64                                          weight streaming
+//   M <= 64                                          weight streaming (M > 32 and N/128 about the unit count: the
+//                                                    kernel that shares the activation block in the workgroup)
 //   few 256x256 tiles, long K                        stream-K (the plain loop would leave most units idle)
 //   128x128 tiles fit one round of two per unit and
 //     (few 256x256 tiles or a short K)               128x128 tiles, K shared between workgroups when they are few
 //   otherwise                                        256x256 ping-pong tiles
 static int pick_variant(int64_t M, int64_t N, int64_t K, int cus) {
+    if (xshare_pays(M, N, K, cus)) return MI355_GEMM_SKINNY_XSHARE;
     if (M <= 64) return MI355_GEMM_SKINNY;
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
@@ -276,6 +333,10 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
         return splits > 1 ? tile128_workspace(M, N, splits) : 0;
     }
     if (variant == MI355_GEMM_TILE256) return MI355_WS_COUNTER_BYTES;  // the tile counters of the persistent launch
+    if (variant == MI355_GEMM_SKINNY_XSHARE) {
+        const int splits = xshare_splits(N, K, cus);
+        return splits > 1 ? xshare_workspace(N, splits) : 0;
+    }
     if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
     const SkinnyPlan pl = skinny_plan(M, N, K, cus);
     return pl.splits > 1 ? skinny_workspace(M, pl) : 0;
@@ -300,7 +361,8 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
                       // 32-bit byte offsets inside a tile / scale column
                       256 * lda < (1ll << 32) && 256 * ldb_n < (1ll << 32) && 256 * as_m * 4 < (1ll << 32) &&
                       as_m >= 0 && as_k >= 0;
-    if (variant == MI355_GEMM_AUTO) {
+    const bool was_auto = variant == MI355_GEMM_AUTO;
+    if (was_auto) {
         variant = fast ? pick_variant(M, N, K, cus) : MI355_GEMM_GENERIC;
         // stream-K needs its partial-tile slots; without them the plain tile loop gives the same result
         if (variant == MI355_GEMM_TILE256_STREAMK &&
@@ -308,6 +370,9 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
             variant = MI355_GEMM_TILE256;
         // the stream kernel's own limits are not errors under AUTO: the 128x128 tile takes every fast layout
         // and runs unsplit without a workspace
+        if (variant == MI355_GEMM_SKINNY_XSHARE &&
+            (N * ldb_n >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)))
+            variant = MI355_GEMM_TILE128;
         if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
             variant = MI355_GEMM_TILE128;
     }
@@ -370,6 +435,17 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
             a.counters = (uint32_t *)ws;
             a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
             return launch_tile<128, 128, 2, 2, 2, kSplitK>(a, a.total_tiles * splits, st);
+        }
+        case MI355_GEMM_SKINNY_XSHARE: {
+            if (M <= 32 || M > 64) return MI355_EUNSUPPORTED;
+            if (N * ldb_n >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)) return MI355_EUNSUPPORTED;
+            if ((N + XshareCfg::BN - 1) / XshareCfg::BN * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
+            int splits = xshare_splits(N, K, cus);
+            if (splits > 1 && (!ws || ws_bytes < xshare_workspace(N, splits) || ((uintptr_t)ws & 15))) {
+                if (was_auto) splits = 1;  // the table's choice runs unsplit without a workspace
+                else return MI355_EWORKSPACE;
+            }
+            return launch_xshare(a, splits, ws, st);
         }
         case MI355_GEMM_SKINNY: {
             const int ok = skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes);
@@ -454,9 +530,9 @@ extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts,
     if (avg <= 16) return 16;
     if (avg <= 32) return 32;
     if (avg <= 64) return 64;
-    // prefill-size batches: the 256x256 ping-pong tile (it skips the empty 64-row halves of ragged blocks);
-    // it needs the activation scales in chunks of 8 K steps
-    return (K / kBlockK) % 8 == 0 ? 256 : 128;
+    // prefill-size batches: the 256x256 ping-pong tile (it skips the empty 64-row halves of ragged blocks)
+    (void)K;
+    return 256;
 }
 
 extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,

@@ -219,6 +219,34 @@ def test_stream_kernel_random_shapes(hip):
         assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
 
 
+def test_shared_activation_stream_kernel(hip):
+    """The streaming kernel whose workgroup shares the activation block (M = 33..64): random shapes with N tails that
+    cut a wave's rows, a workgroup's rows and the vector stores, K from one step to 128, against the torch fp32
+    dequant-matmul, the first streaming kernel (same products, same order per output: bit-equal) and the float64
+    oracle; and the shape the table sends there (N/128 about the number of compute units)."""
+    rng = np.random.default_rng(815)
+    cases = [(int(rng.integers(33, 65)), int(rng.integers(1, 300)) * int(rng.choice([1, 8, 16, 128])),
+              int(rng.choice([128, 384, 1024, 4096, 7168, 16384]))) for _ in range(14)] + [(64, 28672, 4096), (40, 24576, 1536)]
+    for case, (M, N, K) in enumerate(cases):
+        print(f"gemm shared-activation stream case {case}: M={M} N={N} K={K}", flush=True)
+        xq, xs, wq, ws = _prep(M, N, K, seed=5000 + case, device="cuda")
+        c = _run(xq, xs, wq, ws, "xshare")
+        assert not torch.isnan(c.float()).any()
+        ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+        cos, rel = H.gemm_metrics(c.float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (M, N, K, cos, rel)
+        if K <= 2048:   # the first kernel adds a wave's K steps first and the four waves' sums after: same only for few steps
+            assert (c.float() - _run(xq, xs, wq, ws, "skinny").float()).abs().max() <= ref.abs().max() * 2 ** -7
+        rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 4)])
+        cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 30)])
+        ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                              ws.cpu().numpy(), np.arange(len(rows)), cols)
+        got = c[rows][:, cols].float().cpu().double().numpy()
+        assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
+    xq, xs, wq, ws = _prep(64, 28672, 4096, seed=77, device="cuda")
+    assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), _run(xq, xs, wq, ws, "xshare").view(torch.int16))
+
+
 def test_unit_scales_is_plain_matmul(hip):
     """All scales 1: the result is the plain product of the fp8 values, exact in fp32 for K=128."""
     print("gemm unit scales", flush=True)

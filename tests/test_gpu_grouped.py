@@ -142,10 +142,11 @@ def test_grouped_vs_oracle(hip, block_m, mul_w, topk):
 
 @pytest.mark.parametrize("mul_w,topk,T,E", [(False, 4, 200, 7), (True, 1, 900, 5), (False, 2, 40, 9)])
 def test_grouped_256_row_blocks_vs_oracle(hip, mul_w, topk, T, E):
-    """The 256x256 ping-pong tile in grouped mode (needs K % 1024 == 0): experts with fewer than 64, 64-128,
+    """The 256x256 ping-pong tile in grouped mode: experts with fewer than 64, 64-128,
     128-256 and more than 256 rows, so that every combination of skipped half tiles occurs; N tail (640 % 256)."""
     print(f"grouped block_m=256 mul_w={mul_w} topk={topk} T={T} E={E}", flush=True)
     _grouped_case(T=T, E=E, topk=topk, N=640, K=2048, block_m=256, mul_w=mul_w, seed=75)
+    _grouped_case(T=T, E=E, topk=topk, N=640, K=1152, block_m=256, mul_w=mul_w, seed=76)   # K/128 = 9: partial scale chunk
 
 
 def test_grouped_persistent_launch_matches_one_workgroup_per_tile(hip, monkeypatch):
@@ -206,7 +207,7 @@ def test_grouped_random_shapes(hip):
         topk = int(rng.integers(1, min(E, 4) + 1))
         N = int(rng.integers(1, 12)) * 64 + int(rng.choice([0, 8, 40]))
         K = int(rng.choice([128, 384, 1024, 2048]))
-        blocks = [16, 32, 64, 128] + ([256] if K % 1024 == 0 else [])
+        blocks = [16, 32, 64, 128, 256]
         block_m = int(rng.choice(blocks))
         mul_w = bool(rng.integers(0, 2)) and topk == 1
         print(f"grouped random case {case}: T={T} E={E} topk={topk} N={N} K={K} block_m={block_m} mul_w={mul_w}", flush=True)
