@@ -46,7 +46,7 @@ def test_pure_host_entry_points():
     assert lib.mi355_moe_align2_rows(100, 4, 16) == 10
     assert lib.mi355_moe_align2_rows(8, 10, 16) == 8
     assert lib.mi355_grouped_block_m(32768, 256, 4096, 7168) == 256
-    assert lib.mi355_grouped_block_m(32768, 256, 4096, 7168 + 128) == 128
+    assert lib.mi355_grouped_block_m(32768, 256, 4096, 7168 + 128) == 256   # any K/128 takes the 256-row blocks
     assert lib.mi355_grouped_block_m(64, 256, 4096, 7168) == 16
     assert lib.mi355_block_fp8_gemm_workspace_bytes(4096, 4096, 4096, 0) == 65536  # large M: tile counters only
     assert lib.mi355_block_fp8_gemm_workspace_bytes(8, 4096, 14336, 0) > 65536
