@@ -221,6 +221,16 @@ int mi355_silu_and_mul(const void *in, void *out, int64_t M, int64_t H, int64_t 
                        void *stream);
 
 /*
+ * The other forms of the same reference kernel (moe_silu_and_mul.py:46-71): `interleaved` input
+ * [gate0, up0, gate1, up1, ...] instead of [gate | up], and with `use_limit`
+ *     g = min(gate, limit); u = clamp(up, -limit, limit)  (u stays bf16: the bound is limit rounded to bf16)
+ *     out = bf16( bf16(u + 1) * bf16( g / (1 + exp(-g * alpha)) ) ).
+ * Without either flag this is mi355_silu_and_mul.  The reference holds no test of these forms.
+ */
+int mi355_silu_and_mul_ex(const void *in, void *out, int64_t M, int64_t H, int64_t in_stride_m, int64_t out_stride_m,
+                          int32_t interleaved, int32_t use_limit, float limit, float alpha, void *stream);
+
+/*
  * The same product, quantized on the fly: q e4m3fn [M, H] contiguous and one fp32 scale per 1x128 group at
  * s[m * s_stride_m + g * s_stride_g]; arithmetic of mi355_group_quant_fp8 with eps = 1e-10 applied to the bf16
  * products, so the result equals mi355_silu_and_mul followed by mi355_group_quant_fp8 byte for byte.

@@ -46,6 +46,7 @@ SIGNATURES = {
          _c.c_size_t, _vp],
     ),
     "mi355_silu_and_mul": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "mi355_silu_and_mul_ex": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _f32, _f32, _vp]),
     "mi355_silu_and_mul_group_quant_fp8": (
         _c.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i64, _i64, _vp, _i64, _vp]
     ),

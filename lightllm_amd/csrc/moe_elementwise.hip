@@ -22,6 +22,7 @@
 // stand-alone quantizer's code, so its bytes and scales equal those of silu_and_mul followed by the group
 // quantizer.
 #include "quant_core.hpp"
+#include <string.h>
 
 namespace mi355 {
 
@@ -112,6 +113,42 @@ __global__ __launch_bounds__(256) void silu_and_mul_scalar_kernel(const uint16_t
     int64_t row = i / H, col = i - row * H;
     uint32_t g = in[row * in_stride_m + col], u = in[row * in_stride_m + H + col];
     out[row * out_stride_m + col] = (uint16_t)(silu_mul_pk(g, u) & 0xffffu);
+}
+
+// The other forms of the reference kernel (moe_silu_and_mul.py:46-71): "interleaved" input [g0, u0, g1, u1, ...]
+// and the clamped variant  g = min(g, limit); u = clamp(u, -limit, limit);  out = (u + 1) * bf16(g * sigmoid(alpha*g)),
+// where u stays bf16 (so the bound is limit rounded to bf16 and u + 1 is rounded to bf16 before the product).
+// One element per lane: these forms are not on the fp8 block-quantized path.
+__global__ __launch_bounds__(256) void silu_and_mul_general_kernel(const uint16_t *__restrict__ in,
+                                                                   uint16_t *__restrict__ out, int64_t total, int64_t H,
+                                                                   int64_t in_stride_m, int64_t out_stride_m,
+                                                                   int interleaved, int use_limit, float limit,
+                                                                   float limit_bf16, float alpha) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    int64_t row = i / H, col = i - row * H;
+    const uint16_t *r = in + row * in_stride_m;
+    uint32_t gb = interleaved ? r[2 * col] : r[col];
+    uint32_t ub = interleaved ? r[2 * col + 1] : r[H + col];
+    if (!use_limit) {
+        out[row * out_stride_m + col] = (uint16_t)(silu_mul_pk(gb, ub) & 0xffffu);
+        return;
+    }
+    float g = as_f32(gb << 16), u = as_f32(ub << 16);
+    g = g < limit ? g : (g != g ? g : limit);                  // min that keeps a NaN gate
+    u = u > -limit_bf16 ? u : (u != u ? u : -limit_bf16);
+    u = u < limit_bf16 ? u : (u != u ? u : limit_bf16);
+    // 1 / (1 + exp(-g*alpha)) * g, the reference's order of operations
+    const float c1 = 1.44269504088896341f;
+    const float t = g * alpha;
+    const float e = __builtin_amdgcn_exp2f(__builtin_fmaxf(t, -88.0f) * -c1);
+    const float d = 1.0f + e;
+    float rcp = __builtin_amdgcn_rcpf(d);
+    rcp = __builtin_fmaf(__builtin_fmaf(-d, rcp, 1.0f), rcp, rcp);   // one Newton step: 1/d to an ulp
+    const float sg = rcp * g;
+    const float gs = as_f32(f32_to_bf16_bits(sg) << 16);
+    const float up1 = as_f32(f32_to_bf16_bits(u + 1.0f) << 16);
+    out[row * out_stride_m + col] = (uint16_t)f32_to_bf16_bits(up1 * gs);
 }
 
 // One lane = one 8-element chunk of the OUTPUT; 16 lanes (a DPP row) = one quantization group.
@@ -251,6 +288,19 @@ __global__ __launch_bounds__(256) void weight_dequant_scalar_kernel(const uint8_
     out[i] = (uint16_t)f32_to_bf16_bits_nan(a[0] * s[(row >> 7) * kblocks + (col >> 7)]);
 }
 
+// host-side bf16 rounding (nearest even) of the clamp bound
+static inline uint32_t f32_to_bf16_bits_host(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+static inline float as_f32_host(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -278,6 +328,22 @@ extern "C" int mi355_silu_and_mul(const void *in, void *out, int64_t M, int64_t 
         return launch(silu_and_mul_scalar_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, st,
                            (const uint16_t *)in, (uint16_t *)out, total, H, in_stride_m, out_stride_m);
     }
+}
+
+extern "C" int mi355_silu_and_mul_ex(const void *in, void *out, int64_t M, int64_t H, int64_t in_stride_m,
+                                     int64_t out_stride_m, int32_t interleaved, int32_t use_limit, float limit,
+                                     float alpha, void *stream) {
+    if (M < 0 || H < 0) return MI355_EINVAL;
+    if (M == 0 || H == 0) return MI355_OK;
+    if (!in || !out) return MI355_EINVAL;
+    if (in_stride_m < 2 * H || out_stride_m < H) return MI355_ESHAPE;
+    if (!interleaved && !use_limit) return mi355_silu_and_mul(in, out, M, H, in_stride_m, out_stride_m, stream);
+    const int64_t total = M * H;
+    if ((total + 255) / 256 >= (int64_t)1 << 31) return MI355_EUNSUPPORTED;
+    const float limit_bf16 = as_f32_host((uint32_t)f32_to_bf16_bits_host(limit) << 16);
+    return launch(silu_and_mul_general_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                  (const uint16_t *)in, (uint16_t *)out, total, H, in_stride_m, out_stride_m, interleaved ? 1 : 0,
+                  use_limit ? 1 : 0, limit, limit_bf16, alpha);
 }
 
 extern "C" int mi355_silu_and_mul_group_quant_fp8(const void *in, void *q, float *s, int64_t M, int64_t H,

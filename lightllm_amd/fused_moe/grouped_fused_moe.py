@@ -11,7 +11,8 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from ..quantization.fp8act_quant_kernel import per_token_group_quant_fp8
+from ..quantization.fp8act_quant_kernel import lightllm_per_token_group_quant_fp8, per_token_group_quant_fp8
+from .moe_silu_and_mul import silu_and_mul_fwd
 from .moe_silu_and_mul_mix_quant_ep import silu_and_mul_post_quant_fwd
 from .moe_sum_reduce import moe_sum_reduce
 
@@ -208,8 +209,7 @@ def fused_experts_impl(
     """
     assert use_fp8_w8a8 and not use_int8_w8a16, "only the fp8 block-quantized branch is implemented on gfx950"
     assert w1_bias is None and w2_bias is None, "per-expert bias is not supported by the fp8 block branch"
-    if layout != "blocked" or limit is not None or alpha is not None:
-        raise ValueError("fused_experts_impl: only layout='blocked' without limit/alpha is implemented on gfx950")
+    fused_act = layout == "blocked" and limit is None and alpha is None   # else: silu_and_mul_fwd + quantizer
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
@@ -251,7 +251,12 @@ def fused_experts_impl(
             expert_weights=w1, expert_to_weights_scale=w1_scale, topk_num=topk_num, out=c1.view(-1, N),
             mul_routed_weight=False, use_fp8_w8a8=True, alloc_tensor_func=alloc_tensor_func, run_config=run_config,
         )
-        silu_and_mul_post_quant_fwd(c1.view(-1, N), c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128))
+        if fused_act:
+            silu_and_mul_post_quant_fwd(c1.view(-1, N), c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128))
+        else:
+            act = alloc_tensor_func((pairs, N // 2), device=device, dtype=dtype)
+            silu_and_mul_fwd(c1.view(-1, N), act, layout=layout, limit=limit, alpha=alpha)
+            lightllm_per_token_group_quant_fp8(act, 128, c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128))
         grouped_matmul(
             pairs, c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128), expert_to_token_num, expert_to_tokens,
             expert_to_weights=expert_to_weights, expert_weights=w2, expert_to_weights_scale=w2_scale, topk_num=1,

@@ -223,6 +223,16 @@ def silu_and_mul(x_bf16_bits) -> np.ndarray:
     return out
 
 
+def silu_and_mul_ex(x_bf16_bits, layout: str = "blocked", limit=None, alpha=None) -> np.ndarray:
+    x = _c(x_bf16_bits, np.uint16)
+    M, H2 = x.shape
+    out = np.empty((M, H2 // 2), np.uint16)
+    lib().oracle_silu_and_mul_ex(_p(x), I64(M), I64(H2 // 2), I32(1 if layout == "interleaved" else 0),
+                                 I32(0 if limit is None else 1), F32(0.0 if limit is None else limit),
+                                 F32(0.0 if alpha is None else alpha), _p(out))
+    return out
+
+
 def moe_sum_reduce(x_bf16_bits) -> np.ndarray:
     x = _c(x_bf16_bits, np.uint16)
     T, topk, H = x.shape
@@ -246,7 +256,8 @@ def silu_and_mul_group_quant(x_bf16_bits, group: int = 128):
     return group_quant_fp8(silu_and_mul(x_bf16_bits), group)
 
 
-def fused_experts(x_bf16_bits, w1_q, w1_s, w2_q, w2_s, topk_ids, topk_weights) -> np.ndarray:
+def fused_experts(x_bf16_bits, w1_q, w1_s, w2_q, w2_s, topk_ids, topk_weights, layout="blocked", limit=None,
+                  alpha=None) -> np.ndarray:
     """The routed-expert FFN as the reference sequences it (fused_moe/grouped_fused_moe.py:1048-1113):
     routing tables, quantize, gate/up grouped GEMM, silu_and_mul, quantize, down grouped GEMM times the routed
     weight, sum over slots.  x bf16 bits [T,H]; w1 e4m3 bytes [E,2I,H]; w2 [E,H,I] -> bf16 bits [T,H]."""
@@ -257,6 +268,6 @@ def fused_experts(x_bf16_bits, w1_q, w1_s, w2_q, w2_s, topk_ids, topk_weights) -
     idx, ew, cnt = moe_align_fused(ids, topk_weights, E)
     xq, xs = group_quant_fp8(x)
     h1 = grouped_block_gemm(xq, xs, w1_q, w1_s, idx, ew, cnt, topk, False)
-    aq, as_ = silu_and_mul_group_quant(h1)
+    aq, as_ = group_quant_fp8(silu_and_mul_ex(h1, layout, limit, alpha))
     h3 = grouped_block_gemm(aq, as_, w2_q, w2_s, idx, ew, cnt, 1, True)
     return moe_sum_reduce(h3.reshape(T, topk, -1))

@@ -412,6 +412,38 @@ void oracle_silu_and_mul(const uint16_t *in, int64_t M, int64_t H, uint16_t *out
         }
 }
 
+/*
+ * The other forms of the same kernel (moe_silu_and_mul.py:46-71): interleaved input [g0,u0,g1,u1,...] and the
+ * limit/alpha variant
+ *     g = min(gate.f32, limit); u = clamp(up, -limit, limit)    (up stays bf16: the bound is bf16(limit))
+ *     gate = (1 / (1 + exp(-g * alpha)) * g).to(bf16);  out = (u + 1) * gate   (both in bf16 arithmetic)
+ * The reference has no test of these forms: pinned against float64 only ("parity unpinned" by the reference).
+ */
+void oracle_silu_and_mul_ex(const uint16_t *in, int64_t M, int64_t H, int32_t interleaved, int32_t use_limit,
+                            float limit, float alpha, uint16_t *out) {
+    const float lb = oracle_bf16_to_f32(oracle_f32_to_bf16(limit));
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t h = 0; h < H; ++h) {
+            const uint16_t *row = in + m * 2 * H;
+            float g = oracle_bf16_to_f32(interleaved ? row[2 * h] : row[h]);
+            float u = oracle_bf16_to_f32(interleaved ? row[2 * h + 1] : row[H + h]);
+            if (!use_limit) {
+                volatile float sg = g / (1.0f + expf(-g));
+                float gb = oracle_bf16_to_f32(oracle_f32_to_bf16(sg));
+                out[m * H + h] = oracle_f32_to_bf16(gb * u);
+                continue;
+            }
+            if (g > limit) g = limit;
+            if (u < -lb) u = -lb;
+            if (u > lb) u = lb;
+            volatile float sig = 1.0f / (1.0f + expf(-g * alpha));
+            volatile float sg = sig * g;
+            float gb = oracle_bf16_to_f32(oracle_f32_to_bf16(sg));
+            float up1 = oracle_bf16_to_f32(oracle_f32_to_bf16(u + 1.0f));
+            out[m * H + h] = oracle_f32_to_bf16(up1 * gb);
+        }
+}
+
 /* moe_sum_reduce (fused_moe/moe_sum_reduce.py:8-108): out[t,h] = bf16( sum_k in[t,k,h] ), fp32 accumulate
  * in ascending k. */
 void oracle_moe_sum_reduce(const uint16_t *in, int64_t T, int32_t topk, int64_t H, uint16_t *out) {

@@ -40,6 +40,27 @@ def test_fused_experts_vs_oracle(hip, T, E, topk, Hd, I):
     assert (got - want).abs().max() <= 2e-2 * want.abs().max()
 
 
+@pytest.mark.parametrize("layout,limit,alpha", [("interleaved", None, None), ("blocked", 7.0, 1.702), ("interleaved", 7.0, 1.702)])
+def test_fused_experts_other_activation_forms(hip, layout, limit, alpha):
+    """layout / limit / alpha are forwarded to silu_and_mul_fwd as in the reference (grouped_fused_moe.py:1084-1090);
+    the product is then quantized by the stand-alone quantizer instead of the fused kernel."""
+    from lightllm_amd.fused_moe import fused_experts_impl
+
+    print(f"fused_experts layout={layout} limit={limit} alpha={alpha}", flush=True)
+    T, E, topk, Hd, I = 96, 8, 2, 512, 256
+    x = H.activations(T, Hd, seed=41)
+    w1q, w1s, w2q, w2s = _experts(E, I, Hd, seed=43)
+    ids, tw = H.routing(T, E, topk, seed=44)
+    out = fused_experts_impl(x.cuda(), w1q.cuda(), w2q.cuda(), tw.cuda(), ids.cuda(), inplace=False, use_fp8_w8a8=True,
+                             w1_scale=w1s.cuda(), w2_scale=w2s.cuda(), layout=layout, limit=limit, alpha=alpha)
+    torch.cuda.synchronize()
+    want = tr.bf16_from_bits(oracle.fused_experts(tr.bits_of(x), tr.bits_of(w1q), w1s.numpy(), tr.bits_of(w2q),
+                                                  w2s.numpy(), ids.numpy(), tw.numpy(), layout, limit, alpha)).float()
+    got = out.float().cpu()
+    assert tr.cosine(got, want) >= 0.9999
+    assert (got - want).abs().max() <= 2e-2 * want.abs().max()
+
+
 def test_fused_experts_inplace_and_deterministic(hip):
     """Two runs give identical bits (ordered routing tables, no atomics on the output), and inplace writes the
     input tensor (unit_tests/common/fused_moe/test_grouped_fused_moe.py:200-215 checks the same determinism)."""

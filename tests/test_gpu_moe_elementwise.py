@@ -57,15 +57,29 @@ def test_silu_and_mul_extremes_and_strided_input(hip):
     assert torch.isfinite(out.float()).all()
 
 
-def test_silu_and_mul_rejects_other_layouts(hip):
+@pytest.mark.parametrize("layout", ["blocked", "interleaved"])
+@pytest.mark.parametrize("limit,alpha", [(None, None), (7.0, 1.702), (3.3, 1.0)])
+@pytest.mark.parametrize("M,Hh", [(5, 72), (300, 1024)])
+def test_silu_and_mul_other_forms(hip, layout, limit, alpha, M, Hh):
+    """The interleaved layout and the clamped limit/alpha form against the oracle's restatement of
+    moe_silu_and_mul.py:46-71 (the reference holds no vectors for them): within one bf16 ulp on a few elements."""
+    from lightllm_amd.fused_moe import silu_and_mul_fwd
+
+    print(f"silu_and_mul layout={layout} limit={limit} alpha={alpha} M={M} H={Hh}", flush=True)
+    x = (H.activations(M, 2 * Hh, seed=M + Hh + 1).float() * 4).to(torch.bfloat16)
+    out = torch.empty((M, Hh), dtype=torch.bfloat16, device="cuda")
+    silu_and_mul_fwd(x.cuda(), out, layout=layout, limit=limit, alpha=alpha)
+    torch.cuda.synchronize()
+    _silu_close(tr.bits_of(out), oracle.silu_and_mul_ex(tr.bits_of(x), layout, limit, alpha))
+
+
+def test_silu_and_mul_argument_checks(hip):
     from lightllm_amd.fused_moe import silu_and_mul_fwd
 
     x = torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")
     out = torch.empty((4, 128), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(ValueError):
-        silu_and_mul_fwd(x, out, layout="interleaved")
-    with pytest.raises(ValueError):
-        silu_and_mul_fwd(x, out, limit=7.0, alpha=1.7)
+        silu_and_mul_fwd(x, out, layout="rowwise")
     with pytest.raises(AssertionError):
         silu_and_mul_fwd(x, out, limit=7.0)
 

@@ -302,6 +302,40 @@ def test_silu_and_mul_matches_torch_float64_rounding():
     assert (diff != 0).mean() < 1e-3
 
 
+@pytest.mark.parametrize("layout", ["blocked", "interleaved"])
+@pytest.mark.parametrize("limit,alpha", [(None, None), (7.0, 1.702), (3.3, 1.0)])
+def test_silu_and_mul_other_forms_match_float64(layout, limit, alpha):
+    """The interleaved layout and the limit/alpha form (moe_silu_and_mul.py:46-71), against float64 with the same
+    rounding points: gate to bf16, up + 1 to bf16, product to bf16; the clamp bound of `up` is limit rounded to bf16
+    (3.3 is not a bf16 value).  The reference holds no vectors for these forms."""
+    x = (H.activations(48, 512, seed=71).float() * 4).to(torch.bfloat16)
+    xin = x if layout == "blocked" else torch.stack([x[:, :256], x[:, 256:]], dim=-1).reshape(48, 512).contiguous()
+    g, u = x[:, :256].double(), x[:, 256:].double()
+    if limit is None:
+        a = (g / (1 + torch.exp(-g))).float().to(torch.bfloat16)
+        want = (a.float() * u.float()).to(torch.bfloat16)
+    else:
+        lb = float(torch.tensor(limit).to(torch.bfloat16))
+        g = g.clamp(max=float(np.float32(limit)))
+        u = u.clamp(-lb, lb)
+        a = ((1.0 / (1.0 + torch.exp(-(g.float() * np.float32(alpha)).double()))) * g).float().to(torch.bfloat16)
+        want = ((u + 1.0).float().to(torch.bfloat16).float() * a.float()).to(torch.bfloat16)
+    got = oracle.silu_and_mul_ex(tr.bits_of(xin), layout, limit, alpha).astype(np.int32)
+    wantb = tr.bits_of(want).astype(np.int32)
+    diff = np.abs(got - wantb)
+    assert diff.max() <= 1 or np.all((got[diff > 1] & 0x7fff) < 0x80)
+    assert (diff != 0).mean() < 2e-3
+    if limit is None and layout == "blocked":
+        assert np.array_equal(got, oracle.silu_and_mul(tr.bits_of(x)).astype(np.int32))
+    if limit is not None:   # the clamp is active and visible
+        big = torch.full((1, 4), 100.0).to(torch.bfloat16)
+        pair = big if layout == "blocked" else big
+        out = tr.bf16_from_bits(oracle.silu_and_mul_ex(tr.bits_of(pair), layout, limit, alpha)).float()
+        lbv = float(torch.tensor(limit).to(torch.bfloat16))
+        gate = float(np.float32(limit)) / (1.0 + np.exp(-float(np.float32(limit)) * alpha))
+        assert torch.allclose(out, torch.full_like(out, (lbv + 1.0) * gate), rtol=2e-2)
+
+
 def test_moe_sum_reduce_exact_and_ordered():
     # integers: every partial sum is exact, any order gives the same answer
     g = H.gen(71)
