@@ -197,10 +197,13 @@ int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32
  * workspace: optional, used by block_m = 256 only: MI355_WS_COUNTER_BYTES bytes that are zero before the launch
  * (the kernel leaves them zero).  With it the launch is persistent - one workgroup per compute unit takes tiles
  * from per-XCD counters and overlaps the first requests of a tile with the stores of the previous one;
- * without it (NULL) every tile gets its own workgroup, same results.  Launches that may run concurrently
- * need separate workspaces.
+ * without it (NULL) every tile gets its own workgroup, same results.  With mi355_grouped_workspace_bytes(table_rows)
+ * bytes the persistent launch also sorts the schedule rows by size and runs the blocks of at most 64 rows on a
+ * 64x512 weight-streaming tile (same results; the bytes behind the counters are scratch and need no clearing).
+ * Launches that may run concurrently need separate workspaces.
  */
 int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K);
+size_t mi355_grouped_workspace_bytes(int64_t table_rows);
 
 int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,
                                  const int32_t *expert_to_token_index, const float *expert_to_weight,

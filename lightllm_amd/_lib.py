@@ -40,6 +40,7 @@ SIGNATURES = {
     "mi355_moe_align2_rows": (_i64, [_i64, _i32, _i32]),
     "mi355_moe_align2": (_c.c_int, [_vp, _i32, _i32, _i64, _vp, _vp]),
     "mi355_grouped_block_m": (_i32, [_i64, _i32, _i64, _i64]),
+    "mi355_grouped_workspace_bytes": (_sz, [_i64]),
     "mi355_grouped_block_fp8_gemm": (
         _c.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp,

@@ -96,6 +96,16 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xf) | ((N >> 4) << 14) | (0x7 << 4) | (0xf << 8));
 }
 
+// Workgroup barrier that waits for this wave's LDS traffic only (lgkmcnt 0; vmcnt untouched).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8));
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler only: no LDS access may move across the barrier
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);
+}
+
 // 16B-chunk swizzle for LDS tiles with 128-byte rows (8 chunks per row): physical chunk = logical ^ swz(row).
 // For 16 consecutive rows read at one logical chunk the (row parity, physical chunk) pairs are all
 // distinct, and for 8 consecutive rows the physical chunks are all distinct, so a ds_read_b128 of a

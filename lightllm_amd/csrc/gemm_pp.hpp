@@ -36,11 +36,19 @@
 //     most one tile each) and bumps the tile's arrival counter; whoever arrives last adds the tile's partials in K
 //     order (so the result does not depend on who that is), stores the tile and re-zeroes the counter.  Nobody
 //     waits for anybody.
+//   * ROLES (grouped launch with a workspace): schedule blocks with at most 64 rows are weight streams, and this
+//     tile streams badly (32 KiB of W in flight per step, three quarters of the X area and half of the waves
+//     idle).  They go to the 64 x 512 tile of gemm_small.hpp instead, in the same launch: a split kernel has
+//     listed the two kinds of blocks, each kind has its own tile queue, some workgroups start on the small blocks
+//     and the others on the large ones, and a workgroup whose queue is empty moves to the other.  So at any time
+//     part of the device streams weights while the rest computes, where one kind after the other would leave
+//     the matrix cores idle during the streams and the memory idle during the computation.
 //   * SC4: the X scales are row-major with 16-byte aligned rows and K/128 a multiple of 8, and a chunk is fetched
 //     with one 16-byte request per half row.  Otherwise (any strides, any K/128) it is fetched with 4-byte
 //     requests, one per (row, step), four instructions per wave and chunk; steps past the end of K repeat the
 //     last one.
 #pragma once
+#include "gemm_small.hpp"
 #include "gemm_tile.hpp"
 
 namespace mi355 {
@@ -58,36 +66,73 @@ struct PPCfg {
     static constexpr int chunk_off(int KB) { return (kWsOff + 2 * ws_bytes(KB) + 127) & ~127; }
     static constexpr int sched_off(int KB) { return chunk_off(KB) + 2 * kChunkBytes; }
     static constexpr int lds_bytes(int KB) { return sched_off(KB) + 16; }
-    static constexpr int kCounterWords = 9;
+    static constexpr int kCounterWords = 10;          // [0..7] per-XCD tile queues, [8] finished workgroups, [9] small-block queue
+    // ROLES: the LDS word that hands sequence numbers to the waves sits behind both tiles' layouts
+    static constexpr int roles_sched_off(int KB) {
+        return sched_off(KB) > SmallCfg::lds_bytes(KB) ? sched_off(KB) : SmallCfg::lds_bytes(KB);
+    }
     static constexpr int kTileCounterWord = 16;       // stream-K: arrival counters of the tiles start here
     static constexpr int kPartialBytes = BM * BN * 4;  // one fp32 partial tile
 };
 
-template <bool GROUPED, bool SK, bool SC4>
+template <bool GROUPED, bool SK, bool SC4, bool ROLES = false>
 __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p) {
     static_assert(!(GROUPED && SK), "stream-K is a dense launch");
+    static_assert(!ROLES || GROUPED, "the small-block tile belongs to the grouped launch");
     using Cfg = PPCfg;
     constexpr int BM = Cfg::BM, TM = Cfg::TM, TN = Cfg::TN, HM = Cfg::HM, WMS = Cfg::WMS, WNS = Cfg::WNS;
     constexpr bool SKIP = GROUPED;  // ragged tiles skip empty halves; dense tiles keep the branch-free body
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int KB = p.K / kBlockK, nchunk = (KB + 7) >> 3;
+    const uint32_t xcd = blockIdx.x & 7u, in_xcd = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+    const bool persistent = !SK && p.counters != nullptr;
+    volatile uint32_t *sched = (volatile uint32_t *)(lds + (ROLES ? Cfg::roles_sched_off(KB) : Cfg::sched_off(KB)));
+    // ROLES: blocks with more than 64 rows (the tile loop below) and the others (small_blocks), listed by the
+    // split kernel.  The first workgroups of every XCD start on the small blocks, the others on the large ones;
+    // each moves on to the other queue when its own is empty.
+    const int n_big = ROLES ? __builtin_amdgcn_readfirstlane(p.lists[0]) : 0;
+    const int n_small = ROLES ? __builtin_amdgcn_readfirstlane(p.lists[1]) : 0;
+    const int32_t *big_rows = ROLES ? p.lists + 2 : nullptr;
+    const int32_t *small_rows = ROLES ? p.lists + 2 + p.tiles_m : nullptr;
+    const bool small_first = ROLES && in_xcd < (uint32_t)p.small_first;
+    auto small_blocks = [&]() {
+        // one queue for the whole device: (block, pair of n tiles), n fastest
+        const uint32_t pairs_n = (uint32_t)((p.N + SmallCfg::BN - 1) / SmallCfg::BN);
+        const uint32_t total_small = (uint32_t)n_small * pairs_n;
+        while (true) {
+            if (threadIdx.x == 0)
+                sched[0] = __hip_atomic_fetch_add(p.counters + 9, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            const uint32_t item = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
+            __syncthreads();
+            if (item >= total_small) break;
+            const uint32_t blk = item / pairs_n;
+            const v4i row = *(const v4i *)(p.table + (int64_t)small_rows[blk] * 4);
+            grouped_small_tile(p, lds, __builtin_amdgcn_readfirstlane(row[0]), __builtin_amdgcn_readfirstlane(row[1]) * BM,
+                               __builtin_amdgcn_readfirstlane(row[3]), (int)(item - blk * pairs_n) * SmallCfg::BN);
+        }
+    };
+    if constexpr (ROLES) {
+        if (small_first) small_blocks();
+    }
+
+    int tid = threadIdx.x;
+    // ROLES: nothing that depends on the lane is to stay in registers while the other kind of tile runs
+    if constexpr (ROLES) asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave >> 2, wave_n = wave & 3;
     const int grp = wave >> 2;
     const int r16 = lane & 15, g4 = lane >> 4;
     const int sub = lane >> 3;
     const uint32_t pch = (uint32_t)(lane & 7);
-    const int KB = p.K / kBlockK, nchunk = (KB + 7) >> 3;
     const uint32_t lds0 = lds_addr(lds);
-    const uint32_t xcd = blockIdx.x & 7u, in_xcd = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
-    const bool persistent = !SK && p.counters != nullptr;
     // stream-K: this workgroup's run of (tile, K step) units; workgroups are ranked XCD-major so that one XCD works
     // on neighbouring tiles
     const uint32_t rank = xcd * per_xcd + in_xcd;
     const uint64_t units = (uint64_t)p.total_tiles * (uint64_t)KB;
     const uint32_t u_end = SK ? (uint32_t)(((uint64_t)rank + 1u) * units / gridDim.x) : 0u;
-    volatile uint32_t *sched = (volatile uint32_t *)(lds + Cfg::sched_off(KB));
     constexpr uint32_t kNone = 0xffffffffu;
 
     // ---- tile-independent LDS offsets
@@ -129,9 +174,10 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         if (v == kNone) return false;
         if constexpr (GROUPED) {
             const uint64_t bid = (uint64_t)v * 8u + xcd;
-            if (bid >= (uint64_t)p.total_tiles) return false;
+            if (bid >= (ROLES ? (uint64_t)n_big * (uint64_t)p.tiles_n : (uint64_t)p.total_tiles)) return false;
             tile_m = (uint32_t)bid / (uint32_t)p.tiles_n;
             tile_n = (uint32_t)bid - tile_m * (uint32_t)p.tiles_n;
+            if constexpr (ROLES) tile_m = (uint32_t)big_rows[tile_m];
         } else {
             if (v >= (uint32_t)p.blocks_per_xcd) return false;
             const uint32_t logical = xcd * (uint32_t)p.blocks_per_xcd + v;
@@ -305,10 +351,22 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     uint32_t v_next = persistent ? per_xcd + in_xcd : kNone;  // sequence number of the tile after the current one
     uint32_t v_after = kNone;                                 // and of the one after that (fetched)
     uint32_t fetched = 0;
-    const uint32_t v_first = SK ? (uint32_t)((uint64_t)rank * units / gridDim.x) : in_xcd;
-    Tile cur = make_tile(v_first, load_row(in_xcd));
+    uint32_t v_first = SK ? (uint32_t)((uint64_t)rank * units / gridDim.x) : in_xcd;
+    if constexpr (ROLES) {
+        // a workgroup may enter this loop at any time: all its sequence numbers come from the XCD's queue
+        if (tid == 0)
+            for (int i = 0; i < 3; ++i)
+                sched[i] = __hip_atomic_fetch_add(p.counters + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        v_first = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
+        v_next = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[1]);
+        v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[2]);
+        __syncthreads();
+        wsbuf = 0;
+    }
+    Tile cur = make_tile(v_first, load_row(v_first));
     v4i row_next = load_row(v_next);
-    if (persistent && tid == 0)
+    if (!ROLES && persistent && tid == 0)
         fetched = __hip_atomic_fetch_add(p.counters + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // the first requests of a tile: both W slots, the scale chunk(s) of the first steps, X of the first step and
     // the first half of the second
@@ -331,9 +389,9 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         ws_store(cur, 0, ws_load(cur));
     }
     wait_vmcnt<0>();
-    if (persistent && tid == 0) sched[0] = 2u * per_xcd + fetched;
+    if (!ROLES && persistent && tid == 0) sched[0] = 2u * per_xcd + fetched;
     __syncthreads();
-    if (persistent) v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
+    if (!ROLES && persistent) v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
 
     uint32_t u_pos = v_first;  // stream-K: first unit of the current segment
     v4f acc[TM][TN];
@@ -532,10 +590,14 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         wait_vmcnt<0>();
         if (cur.valid) {
             ws_store(cur, wsbuf, ws_first);
-            if (persistent && tid == 0) sched[0] = 2u * per_xcd + fetched;
+            if (persistent && tid == 0) sched[0] = ROLES ? fetched : 2u * per_xcd + fetched;
             __syncthreads();
             if (persistent) v_after = (uint32_t)__builtin_amdgcn_readfirstlane((int)sched[0]);
         }
+    }
+    if constexpr (ROLES) {
+        __syncthreads();  // the other kind of tile lays the LDS out differently
+        if (!small_first) small_blocks();
     }
 
     // ---- the last workgroup to finish leaves the counters zero for the next launch

@@ -63,6 +63,9 @@ struct GemmArgs {
     const int32_t *e_num;        // [E]
     int64_t w_e, ws_e;           // expert strides of W (bytes) and Ws (elements)
     int32_t num_pairs, topk, mul_weight;
+    // grouped launch with two kinds of workgroups (gemm_pp.hpp): row indices of the schedule table split by size
+    const int32_t *lists;        // [0] = blocks with more than 64 rows, [1] = the others, then the two index lists
+    int32_t small_first;         // workgroups per XCD that start on the small blocks
 };
 
 // Which of a wave's 16*TN output columns a lane holds.  The MFMA leaves lane group g (= lane / 16) with the four

@@ -41,16 +41,6 @@ struct ShareCfg {
     static constexpr int scale_lds_bytes(int steps) { return steps * kScaleStride * 4; }
 };
 
-// Workgroup barrier that waits for this wave's LDS traffic only (lgkmcnt 0; vmcnt untouched).
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8));
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);  // compiler only: no LDS access may move across the barrier
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);
-}
-
 template <int MT, int TNW, int DEPTH, bool SPLIT>
 __global__ __launch_bounds__(256) void block_fp8_gemm_xshare_kernel(const GemmArgs p) {
     using Cfg = ShareCfg<MT, TNW, DEPTH>;

@@ -165,7 +165,8 @@ def grouped_matmul(
         table = moe_align2(token_num_mul_topk_num, expert_to_token_num, block_m)
 
     # the 256-row launch is persistent when it gets the (zero at rest) tile counters of this stream's workspace
-    ws = _lib.workspace(out.device, _lib.WS_COUNTER_BYTES) if block_m == 256 else None
+    # (and, given room for the two block lists, runs the blocks of few rows on the weight-streaming tile)
+    ws = _lib.workspace(out.device, lib.mi355_grouped_workspace_bytes(table.shape[0])) if block_m == 256 else None
     code = lib.mi355_grouped_block_fp8_gemm(
         token_inputs.data_ptr(), token_input_scale.data_ptr(), expert_weights.data_ptr(),
         expert_to_weights_scale.data_ptr(), expert_to_token_index.data_ptr(), expert_to_weights.data_ptr(),

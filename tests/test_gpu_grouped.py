@@ -149,6 +149,15 @@ def test_grouped_256_row_blocks_vs_oracle(hip, mul_w, topk, T, E):
     _grouped_case(T=T, E=E, topk=topk, N=640, K=1152, block_m=256, mul_w=mul_w, seed=76)   # K/128 = 9: partial scale chunk
 
 
+@pytest.mark.parametrize("mul_w,topk,T", [(False, 4, 512), (True, 1, 2048)])
+def test_grouped_small_block_tile_tails(hip, mul_w, topk, T):
+    """More tiles than compute units, so the 256-row launch sorts the blocks by size and runs those of at most 64
+    rows on the 64x512 streaming tile: 64 experts with Zipf routing (most blocks small, a few large), an n tail
+    inside the last 512-wide pair (1160 = 2 * 512 + 136), K/128 = 9 (partial scale chunk)."""
+    print(f"grouped small-block tile mul_w={mul_w} topk={topk} T={T}", flush=True)
+    _grouped_case(T=T, E=64, topk=topk, N=1160, K=1152, block_m=256, mul_w=mul_w, seed=77)
+
+
 def test_grouped_persistent_launch_matches_one_workgroup_per_tile(hip, monkeypatch):
     """The 256-row launch with the workspace counters (persistent, tiles handed out per XCD) against the same
     kernel without a workspace (one workgroup per tile): about 600 tiles of mixed cost, identical bits, counter
