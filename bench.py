@@ -229,15 +229,15 @@ def main():
             },
             "roofline": {
                 "bound": "mfma",
-                "kernel": "block_fp8_gemm_pp_kernel<dense> (256x256 tile, persistent)",
+                "kernel": "block_fp8_gemm_pp_kernel<false,false,true,false> (dense 256x256 ping-pong tile, persistent)",
                 "achieved": round(achieved, 1),
                 "peak": FP8_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
                 # HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0), factors from
-                # a 1 GiB device copy: 1692.9 MB read + 311.4 MB written
+                # a 1 GiB device copy: 1695.0 MB read + 311.4 MB written
                 # (profiles/gemm_pp_deepseek_gate_up_M4096.md)
-                "traffic": 2.0043e9,
+                "traffic": 2.0064e9,
                 "algorithmic_bytes_per_launch": gemm_bytes(M, N, K),
                 "launch_us": round(gemm_us, 2),
                 "launch_us_min_max": [round(gemm_all[0], 2), round(gemm_all[-1], 2)],
