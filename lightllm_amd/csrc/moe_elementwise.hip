@@ -33,6 +33,7 @@ __device__ __forceinline__ float silu_f32(float g) {
     const float c2ln2 = 4.888495152e-06f;              // (log2(e) - c1) * ln(2)
     // below -88 the exponential would overflow; silu is below 1e-36 in magnitude from there on, so the
     // argument is held at -88 (the reference gives -0 or a subnormal there)
+    const float gin = g;
     g = __builtin_fmaxf(g, -88.0f);
     float e0 = __builtin_amdgcn_exp2f(g * -c1);
     float e = __builtin_fmaf(e0, g * -c2ln2, e0);      // 2^(hi+lo) ~ 2^hi * (1 + lo*ln2)
@@ -40,7 +41,11 @@ __device__ __forceinline__ float silu_f32(float g) {
     float r = __builtin_amdgcn_rcpf(d);
     float y0 = g * r;
     float res = __builtin_fmaf(-y0, d, g);
-    return __builtin_fmaf(res, r, y0);
+    float out = __builtin_fmaf(res, r, y0);
+    // non-finite gates as g / (1 + exp(-g)) has them: NaN and -inf give NaN (-inf / inf), +inf gives +inf
+    if (__builtin_amdgcn_classf(gin, 0x007)) out = __builtin_nanf("");
+    if (__builtin_amdgcn_classf(gin, 0x200)) out = gin;
+    return out;
 }
 
 // bf16(silu(gate)) * up -> bf16, for the two bf16 values packed in one dword.

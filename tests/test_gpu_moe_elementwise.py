@@ -57,6 +57,34 @@ def test_silu_and_mul_extremes_and_strided_input(hip):
     assert torch.isfinite(out.float()).all()
 
 
+def test_silu_and_mul_non_finite_gates(hip):
+    """gate / (1 + exp(-gate)) of the reference (moe_silu_and_mul.py:33-38): a NaN gate and a -inf gate (-inf / inf)
+    give NaN, a +inf gate gives +inf; products with an infinite or NaN up follow IEEE.  Same NaN positions and the
+    same infinities as the oracle; the other elements as in every other test."""
+    from lightllm_amd.fused_moe import silu_and_mul_fwd
+
+    print("silu_and_mul non-finite", flush=True)
+    M, Hh = 4, 256
+    x = H.activations(M, 2 * Hh, seed=99).clone()
+    x[0, 3] = float("nan")
+    x[0, 40] = float("-inf")
+    x[1, 7] = float("inf")
+    x[1, 8] = float("inf")
+    x[1, Hh + 8] = -1.5               # +inf gate times a negative up
+    x[2, Hh + 100] = float("inf")     # finite gate, infinite up
+    x[3, Hh + 5] = float("nan")
+    out = torch.empty((M, Hh), dtype=torch.bfloat16, device="cuda")
+    silu_and_mul_fwd(x.cuda(), out)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    want = tr.bf16_from_bits(oracle.silu_and_mul(tr.bits_of(x))).float().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(want).sum() >= 3
+    assert np.array_equal(np.isinf(got), np.isinf(want)) and np.isinf(want).sum() >= 3
+    assert np.array_equal(got[np.isinf(want)], want[np.isinf(want)])
+    fin = np.isfinite(want)
+    assert np.abs(got[fin] - want[fin]).max() <= 2 ** -7 * np.abs(want[fin]).max()
+
+
 @pytest.mark.parametrize("layout", ["blocked", "interleaved"])
 @pytest.mark.parametrize("limit,alpha", [(None, None), (7.0, 1.702), (3.3, 1.0)])
 @pytest.mark.parametrize("M,Hh", [(5, 72), (300, 1024)])
@@ -105,6 +133,32 @@ def test_fused_silu_quant_equals_two_steps(hip, M, Hh):
     dq = tr.fp8_from_bits(q_o).float() * torch.from_numpy(s_o).repeat_interleave(128, 1)
     got = q.float().cpu() * s.cpu().repeat_interleave(128, 1)
     assert (got - dq).abs().max() <= 0.07 * dq.abs().max()
+
+
+def test_fused_silu_quant_non_finite_products(hip):
+    """A SiLU product that is NaN or infinite poisons its own 128-element group only, exactly as the stand-alone
+    quantizer does with the bf16 products of silu_and_mul (scale = quiet NaN, bytes = e4m3fn NaN with the sign)."""
+    from lightllm_amd.fused_moe import silu_and_mul_fwd, silu_and_mul_post_quant_fwd
+
+    print("silu+quant non-finite", flush=True)
+    M, Hh = 6, 512
+    x = H.activations(M, 2 * Hh, seed=77).clone()
+    x[1, 5] = float("inf")            # gate +inf: silu = inf, product inf * up
+    x[2, 130] = float("nan")          # gate NaN
+    x[3, Hh + 300] = float("-inf")    # up -inf
+    x[4, 400] = float("-inf")         # gate -inf: silu = -0 * ... (NaN with a finite up only through 0 * inf)
+    x = x.cuda()
+    mid = torch.empty((M, Hh), dtype=torch.bfloat16, device="cuda")
+    silu_and_mul_fwd(x, mid)
+    q = torch.empty((M, Hh), dtype=torch.float8_e4m3fn, device="cuda")
+    s = torch.empty((M, Hh // 128), dtype=torch.float32, device="cuda")
+    silu_and_mul_post_quant_fwd(x, q, s)
+    torch.cuda.synchronize()
+    q_ref, s_ref = oracle.group_quant_fp8(tr.bits_of(mid))
+    assert np.array_equal(tr.bits_of(s), s_ref.view(np.uint32))
+    assert np.array_equal(tr.bits_of(q), q_ref)
+    bad = ~torch.isfinite(mid.float()).cpu().numpy().reshape(M, Hh // 128, 128).all(axis=2)
+    assert bad.sum() >= 4 and np.array_equal(np.isnan(s.cpu().numpy()), bad)
 
 
 def test_fused_silu_quant_column_major_scales(hip):
