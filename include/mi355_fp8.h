@@ -52,7 +52,9 @@ int mi355_device_info(int device, int64_t out[8]);
  * s  fp32, element (m,g) at s[m*s_stride_m + g*s_stride_g], g < K/group
  *    row-major (K/group, 1) and column-major (1, ld) are both what the reference
  *    writes (:37-42); any pair of strides is accepted.
- * group must be 128 and divide K (:80); eps is the floor on the group amax (:55).
+ * group must divide K (:80): 128 is the hot path (16-byte aligned x, 8-byte aligned q), any other size - the whole
+ * row for a per-token scale, as the reference's other callers use it - takes a general kernel; eps is the floor on
+ * the group amax (:55).
  * Arithmetic: s = max(amax,eps)/448 and q = e4m3fn_rtne(clamp(x/s,+-448)) with
  * IEEE fp32 division results, bit for bit.
  * A group that holds a NaN or an infinity (undefined in the reference) gets s = NaN and every byte 0x7F with

@@ -58,7 +58,8 @@ def test_preconditions_are_checked_before_launch():
 
     lib = _lib.lib()
     assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 100, 128, 1e-10, 1, 1, None) == -2   # K % 128
-    assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 256, 64, 1e-10, 4, 1, None) == -6    # group != 128
+    assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 256, 0, 1e-10, 4, 1, None) == -1     # group <= 0
+    assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 256, 96, 1e-10, 4, 1, None) == -2    # K % group
     assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 256, 128, 1e-10, 2, 1, None) == -1   # null
     assert lib.mi355_group_quant_fp8(None, 0, None, None, 0, 256, 128, 1e-10, 2, 1, None) == 0    # empty
     assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 64, 128,

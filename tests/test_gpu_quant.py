@@ -174,3 +174,30 @@ def test_non_finite_groups_are_poisoned(hip, dtype):
     assert np.array_equal(s, s_ref.view(np.uint32))
     assert s[1, 1] == 0x7FC00000 and s[2, 0] == 0x7FC00000 and s[3, 2] == 0x7FC00000 and s[4, 3] == 0x7FC00000
     assert np.all((q[1, 128:256] & 0x7F) == 0x7F) and np.all((q[1, :128] & 0x7F) != 0x7F)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K,group", [(7, 4096, 4096), (33, 14336, 14336), (5, 1024, 64), (9, 768, 256), (4, 120, 24),
+                                       (3, 100, 100), (6, 7168, 512)])
+def test_other_group_sizes(hip, dtype, M, K, group):
+    """The reference's kernel takes any group size that divides K (fp8act_quant_kernel.py:18-60; its other callers
+    quantize per token, group = K): bit-exact against the oracle, groups that are not a multiple of 8 elements and a
+    poisoned group included; column-major scales as well."""
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print(f"quant group={group} {dtype} M={M} K={K}", flush=True)
+    g = H.gen(M + K + group)
+    x = torch.randn((M, K), generator=g, dtype=torch.float32)
+    x[:, ::53] *= 29.0
+    x[1] = 0.0
+    x[2, K // 2] = float("inf")
+    x = x.to(dtype)
+    q_ref, s_ref = oracle.group_quant_fp8_f32(x.float().numpy(), group=group)
+    xq, xs = per_token_group_quant_fp8(x.cuda(), group)
+    torch.cuda.synchronize()
+    assert xs.shape == (M, K // group)
+    assert np.array_equal(tr.bits_of(xs.contiguous()), s_ref.view(np.uint32))
+    assert np.array_equal(tr.bits_of(xq), q_ref)
+    xq2, xs2 = per_token_group_quant_fp8(x.cuda(), group, column_major_scales=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(tr.bits_of(xs2.contiguous()), s_ref.view(np.uint32)) and np.array_equal(tr.bits_of(xq2), q_ref)

@@ -73,6 +73,16 @@ def test_group_quant_equals_torch_closed_form(M, K, kw):
     assert np.array_equal(tr.bits_of(q_t), q_c)
 
 
+@pytest.mark.parametrize("M,K,group", [(4, 4096, 4096), (5, 1024, 64), (3, 120, 24), (2, 100, 100)])
+def test_group_quant_other_group_sizes_equal_torch_closed_form(M, K, group):
+    """The group size is a parameter of the reference's kernel; the oracle follows the same closed form for any."""
+    x = H.activations(M, K, seed=M + K + group, outliers=True)
+    q_t, s_t = tr.group_quant(x, group=group)
+    q_c, s_c = oracle.group_quant_fp8(tr.bits_of(x), group=group)
+    assert np.array_equal(tr.bits_of(s_t), s_c.view(np.uint32))
+    assert np.array_equal(tr.bits_of(q_t), q_c)
+
+
 def test_group_quant_special_cases():
     # all-zero group: eps floor, scale bits of fp32(1e-10)/448, bytes zero
     z = np.zeros((1, 128), np.uint16)
