@@ -147,6 +147,13 @@ int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const fl
                          int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                          int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int32_t block_n,
                          int32_t block_k, void *ws, size_t ws_bytes, int32_t variant, void *stream);
+/* The same with the dtype of C stated: MI355_DTYPE_BF16 or MI355_DTYPE_F16 (the reference casts the accumulator to
+ * whatever C holds, fp8w8a8_block_gemm_kernel.py:78; LightLLM allocates C in the activations' dtype, w8a8.py:515). */
+int mi355_block_fp8_gemm_dtype(const void *A, const void *B, const float *As, const float *Bs, void *C, int64_t M,
+                               int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                               int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int32_t block_n,
+                               int32_t block_k, void *workspace, size_t workspace_bytes, int32_t variant,
+                               int32_t c_dtype, void *stream);
 
 /* ---------------------------------------------------------------------------
  * moe_align_fused / moe_align2 : routing tables for the grouped GEMM
@@ -213,6 +220,14 @@ int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W,
                                  int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
                                  int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
                                  void *workspace, size_t workspace_bytes, void *stream);
+/* The same with the dtype of `out` stated (MI355_DTYPE_BF16 or MI355_DTYPE_F16; `accumulator.to(compute_type)`,
+ * grouped_fused_moe.py:717). */
+int mi355_grouped_block_fp8_gemm_dtype(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                       const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                       const int32_t *expert_token_num, const int32_t *table, int64_t table_rows,
+                                       int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
+                                       int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
+                                       void *ws, size_t ws_bytes, int32_t out_dtype, void *stream);
 
 /* ---- element-wise steps between / after the two expert GEMMs ------------------------------------------------ */
 

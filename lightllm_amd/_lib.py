@@ -34,6 +34,11 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
          _vp, _sz, _i32, _vp],
     ),
+    "mi355_block_fp8_gemm_dtype": (
+        _c.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
+         _vp, _sz, _i32, _i32, _vp],
+    ),
     "mi355_moe_align_fused": (_c.c_int, [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp]),
     "mi355_moe_align": (_c.c_int, [_vp, _i64, _i32, _vp, _i64, _vp]),
     "mi355_moe_align1": (_c.c_int, [_vp, _i64, _vp, _i64, _i32, _vp, _i64, _vp, _vp]),
@@ -45,6 +50,11 @@ SIGNATURES = {
         _c.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp,
          _c.c_size_t, _vp],
+    ),
+    "mi355_grouped_block_fp8_gemm_dtype": (
+        _c.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp,
+         _c.c_size_t, _i32, _vp],
     ),
     "mi355_silu_and_mul": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mi355_silu_and_mul_ex": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _f32, _f32, _vp]),

@@ -23,7 +23,8 @@ __device__ __forceinline__ float e4m3_to_f32(uint8_t b) {
 __global__ __launch_bounds__(256) void block_fp8_gemm_generic_kernel(
     const uint8_t *__restrict__ A, const uint8_t *__restrict__ B, const float *__restrict__ As,
     const float *__restrict__ Bs, uint16_t *__restrict__ C, int M, int N, int K, int64_t lda, int64_t ldb_k,
-    int64_t ldb_n, int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int block_n, int block_k) {
+    int64_t ldb_n, int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int block_n, int block_k,
+    int out_f16) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (int64_t)M * N) return;
     const int m = (int)(idx / N), n = (int)(idx % N);
@@ -35,7 +36,7 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_generic_kernel(
         for (int k = k0; k < k1; ++k) d += e4m3_to_f32(A[m * lda + k]) * e4m3_to_f32(B[k * ldb_k + n * ldb_n]);
         acc += d * As[m * as_m + kb * as_k] * Bs[kb * bs_k + (n / block_n) * bs_n];
     }
-    C[m * ldc + n] = (uint16_t)f32_to_bf16_bits(acc);
+    C[m * ldc + n] = (uint16_t)out_bits(acc, out_f16);
 }
 
 constexpr int kMaxLds = 160 * 1024;  // LDS per workgroup on gfx950
@@ -375,12 +376,14 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     return pl.splits > 1 ? skinny_workspace(M, pl) : 0;
 }
 
-extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C,
-                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
-                                    int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n,
-                                    int32_t block_n, int32_t block_k, void *ws, size_t ws_bytes, int32_t variant,
-                                    void *stream) {
+static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, const float *Bs, void *C, int64_t M,
+                               int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
+                               int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int32_t block_n,
+                               int32_t block_k, void *ws, size_t ws_bytes, int32_t variant, int32_t c_dtype,
+                               void *stream) {
     if (M < 0 || N < 0 || K < 0) return MI355_EINVAL;
+    if (c_dtype != MI355_DTYPE_BF16 && c_dtype != MI355_DTYPE_F16) return MI355_EUNSUPPORTED;
+    const int out_f16 = c_dtype == MI355_DTYPE_F16 ? 1 : 0;
     if (block_n != kBlockN || block_k != kBlockK) return MI355_EUNSUPPORTED;
     if (M == 0 || N == 0) return MI355_OK;
     if (K == 0) return MI355_ESHAPE;
@@ -416,10 +419,11 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
         if (blocks >= (1ll << 31)) return MI355_EUNSUPPORTED;
         return launch(block_fp8_gemm_generic_kernel, dim3((uint32_t)blocks), dim3(256), 0, st, (const uint8_t *)A,
                       (const uint8_t *)B, As, Bs, (uint16_t *)C, (int)M, (int)N, (int)K, lda, ldb_k, ldb_n, ldc, as_m,
-                      as_k, bs_k, bs_n, (int)block_n, (int)block_k);
+                      as_k, bs_k, bs_n, (int)block_n, (int)block_k, out_f16);
     }
 
     GemmArgs a = {};
+    a.out_f16 = out_f16;
     a.X = (const uint8_t *)A;
     a.W = (const uint8_t *)B;
     a.Xs = As;
@@ -493,6 +497,24 @@ extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *A
         default:
             return MI355_EINVAL;
     }
+}
+
+extern "C" int mi355_block_fp8_gemm(const void *A, const void *B, const float *As, const float *Bs, void *C,
+                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n,
+                                    int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n,
+                                    int32_t block_n, int32_t block_k, void *ws, size_t ws_bytes, int32_t variant,
+                                    void *stream) {
+    return block_fp8_gemm_impl(A, B, As, Bs, C, M, N, K, lda, ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n, block_n,
+                               block_k, ws, ws_bytes, variant, MI355_DTYPE_BF16, stream);
+}
+
+extern "C" int mi355_block_fp8_gemm_dtype(const void *A, const void *B, const float *As, const float *Bs, void *C,
+                                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb_k,
+                                          int64_t ldb_n, int64_t ldc, int64_t as_m, int64_t as_k, int64_t bs_k,
+                                          int64_t bs_n, int32_t block_n, int32_t block_k, void *ws, size_t ws_bytes,
+                                          int32_t variant, int32_t c_dtype, void *stream) {
+    return block_fp8_gemm_impl(A, B, As, Bs, C, M, N, K, lda, ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n, block_n,
+                               block_k, ws, ws_bytes, variant, c_dtype, stream);
 }
 
 namespace mi355 {
@@ -572,13 +594,13 @@ extern "C" size_t mi355_grouped_workspace_bytes(int64_t table_rows) {
     return grouped_workspace(table_rows < 0 ? 0 : table_rows);
 }
 
-extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,
-                                            const int32_t *expert_to_token_index, const float *expert_to_weight,
-                                            const int32_t *expert_token_num, const int32_t *table,
-                                            int64_t table_rows, int32_t block_m, int64_t num_pairs,
-                                            int64_t num_tokens, int32_t num_experts, int32_t topk_num, int64_t N,
-                                            int64_t K, int32_t mul_routed_weight, void *out, void *ws,
-                                            size_t ws_bytes, void *stream) {
+static int grouped_block_fp8_gemm_impl(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                       const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                       const int32_t *expert_token_num, const int32_t *table, int64_t table_rows,
+                                       int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
+                                       int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
+                                       void *ws, size_t ws_bytes, int32_t out_dtype, void *stream) {
+    if (out_dtype != MI355_DTYPE_BF16 && out_dtype != MI355_DTYPE_F16) return MI355_EUNSUPPORTED;
     if (num_pairs < 0 || num_tokens < 0 || num_experts <= 0 || topk_num <= 0 || N < 0 || K < 0 || table_rows < 0)
         return MI355_EINVAL;
     if (num_pairs == 0 || N == 0 || table_rows == 0) return MI355_OK;
@@ -593,6 +615,7 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
     const int64_t KB = K / kBlockK, NB = (N + kBlockN - 1) / kBlockN;
 
     GemmArgs a = {};
+    a.out_f16 = out_dtype == MI355_DTYPE_F16 ? 1 : 0;
     a.X = (const uint8_t *)Xq;
     a.W = (const uint8_t *)W;
     a.Xs = Xs;
@@ -637,4 +660,29 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
             return launch_grouped_pp(a, ws, ws_bytes, device_cus(), st);
         default: return MI355_EINVAL;
     }
+}
+
+extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                            const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                            const int32_t *expert_token_num, const int32_t *table,
+                                            int64_t table_rows, int32_t block_m, int64_t num_pairs,
+                                            int64_t num_tokens, int32_t num_experts, int32_t topk_num, int64_t N,
+                                            int64_t K, int32_t mul_routed_weight, void *out, void *ws,
+                                            size_t ws_bytes, void *stream) {
+    return grouped_block_fp8_gemm_impl(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weight, expert_token_num, table,
+                                       table_rows, block_m, num_pairs, num_tokens, num_experts, topk_num, N, K,
+                                       mul_routed_weight, out, ws, ws_bytes, MI355_DTYPE_BF16, stream);
+}
+
+extern "C" int mi355_grouped_block_fp8_gemm_dtype(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                                  const int32_t *expert_to_token_index,
+                                                  const float *expert_to_weight, const int32_t *expert_token_num,
+                                                  const int32_t *table, int64_t table_rows, int32_t block_m,
+                                                  int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
+                                                  int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight,
+                                                  void *out, void *ws, size_t ws_bytes, int32_t out_dtype,
+                                                  void *stream) {
+    return grouped_block_fp8_gemm_impl(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weight, expert_token_num, table,
+                                       table_rows, block_m, num_pairs, num_tokens, num_experts, topk_num, N, K,
+                                       mul_routed_weight, out, ws, ws_bytes, out_dtype, stream);
 }

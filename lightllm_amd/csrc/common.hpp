@@ -35,6 +35,18 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return (uint32_t)__builtin_bit_cast(unsigned short, (__bf16)f);
 }
+// The GEMM outputs: bf16, or fp16 when the caller's tensors are (the reference casts the fp32 accumulator to the
+// dtype of C, quantization/fp8w8a8_block_gemm_kernel.py:78).  `f16` is the same for every lane of a launch.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_out2(float lo, float hi, int f16) {
+    v2f v = {lo, hi};
+    if (f16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t out_bits(float f, int f16) {
+    if (f16) return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
+    return f32_to_bf16_bits(f);
+}
 
 // D(16x16, fp32) = A(16x128, e4m3) * B(128x16, e4m3) + C on the CDNA4 matrix core.
 // Lane l feeds row/col (l % 16) and the 32 K-bytes numbered (l / 16); both operands use the same

@@ -176,13 +176,13 @@ __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *l
 #pragma unroll
             for (int h = 0; h < TN / 2; ++h)
                 *(v4i *)(cp + lane_col<TN>(g4, 2 * h)) =
-                    v4i{(int)pack_bf16x2(o[8 * h + 0], o[8 * h + 1]), (int)pack_bf16x2(o[8 * h + 2], o[8 * h + 3]),
-                        (int)pack_bf16x2(o[8 * h + 4], o[8 * h + 5]), (int)pack_bf16x2(o[8 * h + 6], o[8 * h + 7])};
+                    v4i{(int)pack_out2(o[8 * h + 0], o[8 * h + 1], p.out_f16), (int)pack_out2(o[8 * h + 2], o[8 * h + 3], p.out_f16),
+                        (int)pack_out2(o[8 * h + 4], o[8 * h + 5], p.out_f16), (int)pack_out2(o[8 * h + 6], o[8 * h + 7], p.out_f16)};
         } else {
 #pragma unroll
             for (int e = 0; e < 4 * TN; ++e) {
                 const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
-                if (nbase + c < p.N) cp[c] = (uint16_t)f32_to_bf16_bits(o[e]);
+                if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
             }
         }
     }

@@ -298,11 +298,11 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_stream_kernel(const GemmAr
         if (m >= p.M) continue;
         uint16_t *cp = p.C + (int64_t)m * p.ldc + ncol;
         if (p.vec_store && ncol + 4 <= p.N) {
-            *(v2i *)cp = v2i{(int)pack_bf16x2(sum[q][0], sum[q][1]), (int)pack_bf16x2(sum[q][2], sum[q][3])};
+            *(v2i *)cp = v2i{(int)pack_out2(sum[q][0], sum[q][1], p.out_f16), (int)pack_out2(sum[q][2], sum[q][3], p.out_f16)};
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                if (ncol + e < p.N) cp[e] = (uint16_t)f32_to_bf16_bits(sum[q][e]);
+                if (ncol + e < p.N) cp[e] = (uint16_t)out_bits(sum[q][e], p.out_f16);
         }
     }
 }

@@ -52,6 +52,7 @@ struct GemmArgs {
     int64_t ldx, ldw, ldc;
     int64_t xs_m, xs_k, ws_n, ws_k;
     int32_t vec_store;   // 1: C rows are 16-byte aligned and N % 8 == 0
+    int32_t out_f16;     // 0: C is bf16, 1: C is fp16
     // split-K launch only
     int32_t splits;
     uint32_t *counters;  // [total_tiles], zero before the launch, zero again after it
@@ -443,19 +444,19 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
             for (int v = 0; v < 4; ++v) o[4 * j + v] = GROUPED ? acc[i][j][v] * rw : acc[i][j][v];
         if (p.vec_store && nbase + WNS <= p.N) {
             if constexpr (TN == 1) {
-                *(v2i *)(cp + lane_col<TN>(g4, 0)) = v2i{(int)pack_bf16x2(o[0], o[1]), (int)pack_bf16x2(o[2], o[3])};
+                *(v2i *)(cp + lane_col<TN>(g4, 0)) = v2i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16)};
             } else {
 #pragma unroll
                 for (int h = 0; h < TN / 2; ++h)
                     *(v4i *)(cp + lane_col<TN>(g4, 2 * h)) =
-                        v4i{(int)pack_bf16x2(o[8 * h + 0], o[8 * h + 1]), (int)pack_bf16x2(o[8 * h + 2], o[8 * h + 3]),
-                            (int)pack_bf16x2(o[8 * h + 4], o[8 * h + 5]), (int)pack_bf16x2(o[8 * h + 6], o[8 * h + 7])};
+                        v4i{(int)pack_out2(o[8 * h + 0], o[8 * h + 1], p.out_f16), (int)pack_out2(o[8 * h + 2], o[8 * h + 3], p.out_f16),
+                            (int)pack_out2(o[8 * h + 4], o[8 * h + 5], p.out_f16), (int)pack_out2(o[8 * h + 6], o[8 * h + 7], p.out_f16)};
             }
         } else {
 #pragma unroll
             for (int e = 0; e < 4 * TN; ++e) {
                 const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
-                if (nbase + c < p.N) cp[c] = (uint16_t)f32_to_bf16_bits(o[e]);
+                if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
             }
         }
     }

@@ -255,17 +255,17 @@ __global__ __launch_bounds__(256) void block_fp8_gemm_xshare_kernel(const GemmAr
         uint16_t *cp = p.C + (int64_t)m * p.ldc + nw + 4 * TNW * g4;
         if (p.vec_store && nw + 16 * TNW <= p.N) {
             if constexpr (TNW == 2) {
-                *(v4i *)cp = v4i{(int)pack_bf16x2(acc[t][0][0], acc[t][0][1]), (int)pack_bf16x2(acc[t][0][2], acc[t][0][3]),
-                                 (int)pack_bf16x2(acc[t][1][0], acc[t][1][1]), (int)pack_bf16x2(acc[t][1][2], acc[t][1][3])};
+                *(v4i *)cp = v4i{(int)pack_out2(acc[t][0][0], acc[t][0][1], p.out_f16), (int)pack_out2(acc[t][0][2], acc[t][0][3], p.out_f16),
+                                 (int)pack_out2(acc[t][1][0], acc[t][1][1], p.out_f16), (int)pack_out2(acc[t][1][2], acc[t][1][3], p.out_f16)};
             } else {
-                *(v2i *)cp = v2i{(int)pack_bf16x2(acc[t][0][0], acc[t][0][1]), (int)pack_bf16x2(acc[t][0][2], acc[t][0][3])};
+                *(v2i *)cp = v2i{(int)pack_out2(acc[t][0][0], acc[t][0][1], p.out_f16), (int)pack_out2(acc[t][0][2], acc[t][0][3], p.out_f16)};
             }
         } else {
 #pragma unroll
             for (int j = 0; j < TNW; ++j)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (nw + 4 * TNW * g4 + 4 * j + e < p.N) cp[4 * j + e] = (uint16_t)f32_to_bf16_bits(acc[t][j][e]);
+                    if (nw + 4 * TNW * g4 + 4 * j + e < p.N) cp[4 * j + e] = (uint16_t)out_bits(acc[t][j][e], p.out_f16);
         }
     }
 }

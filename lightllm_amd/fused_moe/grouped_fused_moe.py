@@ -142,7 +142,7 @@ def grouped_matmul(
     assert expert_to_weights_scale.shape[1] == (n + 127) // 128 and expert_to_weights_scale.shape[2] * 128 == k, (
         "weights must be 128x128 block-quantized"
     )
-    assert out.dtype == torch.bfloat16 and out.shape[1] == n
+    assert out.dtype in (torch.bfloat16, torch.float16) and out.shape[1] == n
     _lib.require_cuda(token_inputs, expert_weights, out)
     lib = _lib.lib()
 
@@ -167,12 +167,13 @@ def grouped_matmul(
     # the 256-row launch is persistent when it gets the (zero at rest) tile counters of this stream's workspace
     # (and, given room for the two block lists, runs the blocks of few rows on the weight-streaming tile)
     ws = _lib.workspace(out.device, lib.mi355_grouped_workspace_bytes(table.shape[0])) if block_m == 256 else None
-    code = lib.mi355_grouped_block_fp8_gemm(
+    code = lib.mi355_grouped_block_fp8_gemm_dtype(
         token_inputs.data_ptr(), token_input_scale.data_ptr(), expert_weights.data_ptr(),
         expert_to_weights_scale.data_ptr(), expert_to_token_index.data_ptr(), expert_to_weights.data_ptr(),
         expert_to_token_num.data_ptr(), table.data_ptr(), table.shape[0], block_m, token_num_mul_topk_num,
         token_inputs.shape[0], expert_num, topk_num, n, k, 1 if mul_routed_weight else 0, out.data_ptr(),
-        ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _lib.stream_ptr(out.device),
+        ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _lib.DTYPE_CODES[out.dtype],
+        _lib.stream_ptr(out.device),
     )
     _lib.check(code, "grouped_matmul")
     return (table, block_m)

@@ -56,7 +56,7 @@ def _launch(x, xs, w, ws, out, index, counts, rows, stride, E, N, K, block_m=Non
         block_m = lib.mi355_grouped_block_m(rows, E, N, K)
     assert block_m in _BLOCK_MS
     table = moe_align2(rows, counts, block_m)
-    wsp = _lib.workspace(out.device, _lib.WS_COUNTER_BYTES) if block_m == 256 else None
+    wsp = _lib.workspace(out.device, lib.mi355_grouped_workspace_bytes(table.shape[0])) if block_m == 256 else None
     code = lib.mi355_grouped_block_fp8_gemm(
         x.data_ptr(), xs.data_ptr(), w.data_ptr(), ws.data_ptr(), index.data_ptr(), xs.data_ptr(), counts.data_ptr(),
         table.data_ptr(), table.shape[0], block_m, stride, rows, E, 1, N, K, 0, out.data_ptr(),

@@ -49,7 +49,7 @@ def w8a8_block_fp8_matmul(
     assert _cdiv(K, block_k) == Ascale.shape[-1] and Ascale.shape[-1] == Bscale.shape[0]
     assert _cdiv(N, block_n) == Bscale.shape[1]
     assert C.shape[0] == M and C.shape[1] == N
-    assert C.dtype == torch.bfloat16 and dtype == torch.bfloat16, "the gfx950 kernels write bf16"
+    assert C.dtype in (torch.bfloat16, torch.float16), "the gfx950 kernels write bf16 or fp16"
     assert A.dtype == torch.float8_e4m3fn and B.dtype == torch.float8_e4m3fn
     assert Ascale.dtype == torch.float32 and Bscale.dtype == torch.float32
     _lib.require_cuda(A, B, Ascale, Bscale, C)
@@ -62,11 +62,12 @@ def w8a8_block_fp8_matmul(
     if need:
         ws = _lib.workspace(A.device, need)
         ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
-    code = lib.mi355_block_fp8_gemm(
+    # the accumulator is cast to the dtype of C, like `accumulator.to(C.dtype.element_ty)` in the reference (:78)
+    code = lib.mi355_block_fp8_gemm_dtype(
         A.data_ptr(), B.data_ptr(), Ascale.data_ptr(), Bscale.data_ptr(), C.data_ptr(), M, N, K,
         A.stride(0), B.stride(0), B.stride(1), C.stride(0),
         Ascale.stride(0), Ascale.stride(1), Bscale.stride(0), Bscale.stride(1),
-        block_n, block_k, ws_ptr, ws_bytes, variant, _lib.stream_ptr(A.device),
+        block_n, block_k, ws_ptr, ws_bytes, variant, _lib.DTYPE_CODES[C.dtype], _lib.stream_ptr(A.device),
     )
     _lib.check(code, "w8a8_block_fp8_matmul")
     return C

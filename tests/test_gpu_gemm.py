@@ -416,3 +416,44 @@ def test_quant_method_apply(hip):
     xq, xs = per_token_group_quant_fp8(x, 128)
     C = _run(xq, xs, pack.weight, pack.weight_scale)
     assert torch.equal(C, out)
+    # an fp16 model: fp16 activations are quantized as they are and the output comes back in fp16 (w8a8.py:507-529)
+    x16 = x.to(torch.float16)
+    out16 = method.apply(x16, pack)
+    torch.cuda.synchronize()
+    assert out16.dtype == torch.float16 and out16.shape == (40, 768)
+    assert tr.cosine(out16.float(), ref) > 0.999
+
+
+@pytest.mark.parametrize("variant,M,N,K", [("tile256", 300, 1000, 1152), ("tile256once", 512, 512, 1024), ("tile128", 130, 520, 512),
+                                           ("tile256x128", 260, 300, 256), ("skinny", 9, 1000, 2048), ("skinny", 40, 4100, 4096),
+                                           ("xshare", 50, 4096, 1024), ("tile256streamk", 1000, 2048, 16384),
+                                           ("generic", 7, 130, 256), (None, 64, 28672, 4096), (None, 1024, 2112, 7168)])
+def test_fp16_output(hip, variant, M, N, K):
+    """C in fp16: the fp32 accumulator is cast to the dtype of C (fp8w8a8_block_gemm_kernel.py:78; LightLLM allocates C
+    in the activations' dtype).  Every kernel against the same launch with bf16 output - the fp16 values must be the
+    fp16 rounding of a number whose bf16 rounding is the bf16 result - and against the float64 oracle on a sample."""
+    print(f"gemm fp16 out variant={variant} M={M} N={N} K={K}", flush=True)
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + N + K)
+    c16 = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    from lightllm_amd.quantization import w8a8_block_fp8_matmul
+
+    w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), c16, [128, 128], dtype=torch.float16,
+                          run_config={"variant": variant} if variant else None)
+    torch.cuda.synchronize()
+    cb = _run(xq, xs, wq, ws, variant)
+    assert not torch.isnan(c16.float()).any()
+    # same accumulator, two roundings: they agree to bf16 precision, and fp16 is the finer one
+    assert (c16.float() - cb.float()).abs().max() <= 2 ** -8 * cb.float().abs().max()
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(c16.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+    e16 = (c16.float() - ref).abs().mean()
+    eb = (cb.float() - ref).abs().mean()
+    assert e16 <= eb, (float(e16), float(eb))   # three more mantissa bits than bf16
+    rng = np.random.default_rng(M)
+    rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 4)])
+    cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 30)])
+    ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                          ws.cpu().numpy(), np.arange(len(rows)), cols)
+    got = c16[rows][:, cols].float().cpu().double().numpy()
+    assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * np.abs(ref64).max()

@@ -284,3 +284,43 @@ def test_grouped_deepseek_shape_sampled(hip, block_m):
         ref = dx[rows // topk] @ tr.dequant(wq[e], ws[e], 128, 128).T
         cos, rel = H.gemm_metrics(out[rows].float(), ref)
         assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (e, cos, rel)
+
+
+@pytest.mark.parametrize("block_m", [16, 64, 128, 256])
+def test_grouped_fp16_output(hip, block_m):
+    """out in fp16 (`accumulator.to(compute_type)`, grouped_fused_moe.py:717): every row-block size, the 256-row launch
+    with enough tiles for the small-block tile; against the bf16 launch and the torch fp32 dequant-matmul per expert."""
+    from lightllm_amd.fused_moe import grouped_matmul
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print(f"grouped fp16 out block_m={block_m}", flush=True)
+    T, E, topk, N, K = 700, 40, 4, 1160, 1152
+    ids, tw = H.routing(T, E, topk, seed=31)
+    idx, w, cnt = _align(ids, tw, E)
+    x = H.activations(T, K, seed=32).cuda()
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, -(-N // 128), K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=300 + e, device="cuda")
+    P = T * topk
+    outs = {}
+    for dt in (torch.float16, torch.bfloat16):
+        out = torch.full((P, N), float("nan"), dtype=dt, device="cuda")
+        grouped_matmul(P, xq, xs, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=True, use_fp8_w8a8=True,
+                       run_config={"BLOCK_SIZE_M": block_m})
+        torch.cuda.synchronize()
+        assert not torch.isnan(out.float()).any()
+        outs[dt] = out
+    a, b = outs[torch.float16].float(), outs[torch.bfloat16].float()
+    assert (a - b).abs().max() <= 2 ** -8 * b.abs().max()
+    cnt_h, idx_h, w_h = cnt.cpu(), idx.cpu(), w.cpu()
+    for e in range(0, E, 7):
+        n_e = int(cnt_h[e])
+        if n_e == 0:
+            continue
+        pairs = idx_h[e, :n_e].long().cuda()
+        ref = tr.dequant_matmul(xq[pairs // topk], xs[pairs // topk], wq[e], ws[e], out_dtype=torch.float32)
+        ref = ref * w_h[e, :n_e].cuda()[:, None]
+        cos, rel = H.gemm_metrics(a[pairs], ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (e, cos, rel)
