@@ -158,6 +158,58 @@ def test_grouped_small_block_tile_tails(hip, mul_w, topk, T):
     _grouped_case(T=T, E=64, topk=topk, N=1160, K=1152, block_m=256, mul_w=mul_w, seed=77)
 
 
+@pytest.mark.parametrize("T,E,topk,what", [(1500, 40, 1, "only small blocks"), (3000, 6, 2, "only large blocks"),
+                                           (2100, 30, 1, "blocks of exactly 64 and 65 rows")])
+def test_grouped_two_queues_degenerate(hip, T, E, topk, what):
+    """The launch with two work queues when one of them is empty, and at the boundary between them: uniform routing
+    (zipf_s = 0) gives every expert about the same count; the third case forces counts of 64, 65, 128 and 129 rows.
+    N = 3072 makes more tiles than compute units in every case."""
+    from lightllm_amd.fused_moe import grouped_matmul, moe_align_fused
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print(f"grouped two queues: {what}", flush=True)
+    N, K = 3072, 512
+    if "exactly" in what:
+        counts = ([64, 65, 128, 129, 1, 63] * 5)[:E]
+        ids = torch.cat([torch.full((c,), e, dtype=torch.int32) for e, c in enumerate(counts)])
+        T = ids.numel()
+        ids = ids[torch.randperm(T, generator=H.gen(3))].reshape(T, 1).contiguous()
+        tw = torch.rand((T, 1), generator=H.gen(4)).float()
+    else:
+        ids, tw = H.routing(T, E, topk, seed=41, zipf_s=0.0)
+    P = T * topk
+    idx = torch.empty((E, P), dtype=torch.int32, device="cuda")
+    w = torch.empty((E, P), dtype=torch.float32, device="cuda")
+    cnt = torch.empty((E,), dtype=torch.int32, device="cuda")
+    moe_align_fused(idx, w, cnt, ids.cuda(), tw.cuda())
+    counts_h = cnt.cpu().numpy()
+    if "small" in what:
+        assert counts_h.max() <= 64
+    if "large" in what:
+        assert counts_h.min() > 64
+    x = H.activations(T, K, seed=42).cuda()
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, N // 128, K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=500 + e, device="cuda")
+    out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    grouped_matmul(P, xq, xs, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=True, use_fp8_w8a8=True,
+                   run_config={"BLOCK_SIZE_M": 256})
+    torch.cuda.synchronize()
+    assert not torch.isnan(out.float()).any(), "a routed row was not written"
+    idx_h, w_h = idx.cpu(), w.cpu()
+    for e in range(E):
+        n_e = int(counts_h[e])
+        if n_e == 0:
+            continue
+        pairs = idx_h[e, :n_e].long().cuda()
+        ref = tr.dequant_matmul(xq[pairs // topk], xs[pairs // topk], wq[e], ws[e], out_dtype=torch.float32)
+        ref = ref * w_h[e, :n_e].cuda()[:, None]
+        cos, rel = H.gemm_metrics(out[pairs].float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (e, n_e, cos, rel)
+
+
 def test_grouped_persistent_launch_matches_one_workgroup_per_tile(hip, monkeypatch):
     """The 256-row launch with the workspace counters (persistent, tiles handed out per XCD) against the same
     kernel without a workspace (one workgroup per tile): about 600 tiles of mixed cost, identical bits, counter
