@@ -62,7 +62,7 @@ def test_grouped_gemm_under_graph_capture(hip):
     from lightllm_amd.quantization import per_token_group_quant_fp8
 
     print("graph capture grouped gemm", flush=True)
-    T, E, topk, N, K = 1536, 12, 4, 2048, 1024
+    T, E, topk, N, K = 1536, 24, 4, 4096, 1024       # more tiles than compute units: persistent, both work queues
     ids, tw = H.routing(T, E, topk, seed=15)
     P = T * topk
     idx = torch.empty((E, P), dtype=torch.int32, device="cuda")
