@@ -1,0 +1,289 @@
+// Block-scaled FP8 GEMM for 65..128 activation rows on gfx950: a weight stream with the activation block in LDS.
+//
+// With at most 128 rows of X every weight byte is used once per launch, so the launch is a stream over W, and the
+// square tiles spend it badly: a 128x128 tile keeps 16 KiB of W per K step in flight and one round of such tiles
+// is bound by the latency of its steps, not by the memory.  This kernel is the 64-row tile of the grouped GEMM
+// (gemm_small.hpp) with twice the rows and a dense epilogue:
+//
+//   16*MT activation rows (MT = 5..8 MFMA row blocks) x 256 weight rows, K step 128.
+//   8 waves, wave w owns weight rows [32w, 32w+32) and all activation rows: MT x 2 MFMA blocks per K step.
+//   NS ring slots of { X 16*MT x 128 B, W 256 x 128 B }.  A wave fetches its own W rows (4 requests of 1 KiB per
+//   step) into its own part of a slot and is the only one to read them, so the W stream needs no barrier: the rows
+//   of step kb + NS are requested as soon as the wave has read those of step kb.  The X block is shared: one barrier
+//   per step makes step kb visible and frees the slot of step kb - 1 for step kb + NS - 1.
+//   X scales come in [rows][8 steps] chunks by 4-byte requests (any scale layout); the W scales of the tile's two
+//   128-wide n blocks are copied to LDS once.
+//   When N / 256 tiles are too few for the device the K range is shared between workgroups.  Their partial sums
+//   are 16*MT x 256 floats each, too many for the last workgroup of a tile to add alone (one compute unit reads
+//   about 40 GB/s): they go to the workspace and a second, device-wide launch adds them in split order.
+//
+// Arithmetic, operand layouts in LDS and the epilogue are those of the other tiled kernels (gemm_tile.hpp).
+#pragma once
+#include "gemm_tile.hpp"
+
+namespace mi355 {
+
+template <int MT, int NS>
+struct Rows128Cfg {
+    static_assert(MT >= 1 && MT <= 8 && (NS == 2 || NS == 3), "");
+    static constexpr int BN = 256, kWaves = 8, kThreads = 512, TN = 2, WNS = 32;
+    static constexpr int XG = 2 * MT;                          // 8-row request groups of the X block
+    static constexpr int NXW = (XG + kWaves - 1) / kWaves;     // X requests per wave (groups repeat if XG % 8 != 0)
+    static constexpr int kXBytes = 16 * MT * 128, kWBytes = BN * 128;
+    static constexpr int kStage = kXBytes + kWBytes;
+    static constexpr int kWsOff = NS * kStage;                 // W scales [2 n blocks][steps]
+    static constexpr int kChunkBytes = 16 * MT * 32;           // one [rows][8 steps] chunk of X scales
+    static constexpr int kTileElems = 16 * MT * BN;
+    static constexpr int chunk_off(int steps) { return (kWsOff + 2 * steps * 4 + 127) & ~127; }
+    static constexpr int lds_bytes(int steps) { return chunk_off(steps) + 2 * kChunkBytes; }
+};
+
+template <int MT, int NS, bool SPLIT>
+__global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmArgs p) {
+    using Cfg = Rows128Cfg<MT, NS>;
+    constexpr int TN = Cfg::TN, WNS = Cfg::WNS, NXW = Cfg::NXW, XG = Cfg::XG;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, g4 = lane >> 4, sub = lane >> 3;
+    const uint32_t pch = (uint32_t)(lane & 7);
+
+    uint32_t tile_n, split = 0;
+    if constexpr (SPLIT) {
+        tile_n = blockIdx.x / (uint32_t)p.splits;
+        split = blockIdx.x - tile_n * (uint32_t)p.splits;
+    } else {
+        tile_n = blockIdx.x;
+    }
+    const int n0 = (int)tile_n * Cfg::BN;
+    const int KB = p.K / kBlockK;
+    int kb_begin = 0, kb_end = KB;
+    if constexpr (SPLIT) {
+        const int per = KB / p.splits, rem = KB % p.splits;
+        kb_begin = (int)split * per + min((int)split, rem);
+        kb_end = kb_begin + per + ((int)split < rem ? 1 : 0);
+    }
+    const int steps = kb_end - kb_begin;
+    const uint32_t lds0 = lds_addr(lds);
+
+    // ---- request offsets (rows past the matrices are clamped; their results are never stored)
+    uint32_t xoff[NXW], xdst[NXW], sc_row[NXW], sdst[NXW];
+#pragma unroll
+    for (int i = 0; i < NXW; ++i) {
+        const int g = (wave + Cfg::kWaves * i) % XG;  // waves beyond the block repeat a group (same bytes)
+        const int row = 8 * g + sub;
+        const uint32_t src = (uint32_t)min(row, p.M - 1);
+        xoff[i] = src * (uint32_t)p.ldx + (pch ^ swz((uint32_t)row)) * 16u;
+        xdst[i] = (uint32_t)g * 1024u;
+        sc_row[i] = src * (uint32_t)p.xs_m;
+        sdst[i] = (uint32_t)g * 256u;
+    }
+    uint32_t woff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int w = 8 * i + sub;  // LDS row inside the wave's 32-row span
+        const int tn = w >> 4, gg = (w >> 2) & 3, vv = w & 3;
+        const int nl = wave * WNS + lane_col<TN>(gg, tn) + vv;
+        const int nc = min(n0 + nl, p.N - 1) - n0;
+        woff[i] = (uint32_t)nc * (uint32_t)p.ldw + (pch ^ swz((uint32_t)w)) * 16u;
+    }
+    const uint8_t *wg = p.W + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kBlockK;
+    const uint8_t *xg = p.X + (int64_t)kb_begin * kBlockK;
+    const uint32_t wdst = (uint32_t)Cfg::kXBytes + (uint32_t)wave * (WNS * 128u);
+    const uint32_t chunk_off = (uint32_t)Cfg::chunk_off(steps);
+
+    auto issue_w = [&](int slot, int it) {
+        const uint32_t sb = lds0 + (uint32_t)slot * Cfg::kStage + wdst;
+        const uint8_t *wk = wg + (int64_t)it * kBlockK;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma_g2l_b128(sb + (uint32_t)i * 1024u, wk, woff[i]);
+    };
+    auto issue_x = [&](int slot, int it) {
+        const uint32_t sb = lds0 + (uint32_t)slot * Cfg::kStage;
+        const uint8_t *xk = xg + (int64_t)it * kBlockK;
+#pragma unroll
+        for (int i = 0; i < NXW; ++i) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
+    };
+    auto issue_scales = [&](int chunk) {
+        const uint32_t st = (uint32_t)min(lane & 7, steps - 1 - 8 * chunk) * (uint32_t)p.xs_k;
+        const float *base = p.Xs + (int64_t)(kb_begin + 8 * chunk) * p.xs_k;
+#pragma unroll
+        for (int i = 0; i < NXW; ++i)
+            dma_g2l_b32(lds0 + chunk_off + (uint32_t)(chunk & 1) * Cfg::kChunkBytes + sdst[i], base, (sc_row[i] + st) * 4u);
+    };
+
+    // ---- per-lane LDS read offsets
+    const uint32_t fr = swz((uint32_t)r16);
+    const uint32_t c0 = ((uint32_t)(2 * g4)) ^ fr, c1 = c0 ^ 1u;
+    const uint32_t xr0 = (uint32_t)r16 * 128u + c0 * 16u, xr1 = (uint32_t)r16 * 128u + c1 * 16u;
+    const uint32_t wr0 = wdst + xr0, wr1 = wdst + xr1;
+    const uint32_t sr8 = chunk_off + (uint32_t)r16 * 32u;
+
+    // ---- first requests, in the order of the steady state: step j issues X(j+NS-1), its scale chunk, W(j+NS)
+#pragma unroll
+    for (int j = -NS; j < 0; ++j) {
+        const int xi = j + NS - 1, wi = j + NS;
+        if (xi >= 0 && xi < steps) {
+            issue_x(xi % NS, xi);
+            if (xi == 0) issue_scales(0);
+        }
+        if (wi < steps) issue_w(wi % NS, wi);
+    }
+    {
+        const int NBk = (p.N + kBlockN - 1) / kBlockN;
+        float *wl = (float *)(lds + Cfg::kWsOff);
+        for (int i = tid; i < 2 * steps; i += Cfg::kThreads) {
+            const int b = i >= steps ? 1 : 0, it = i - b * steps;
+            wl[i] = p.Ws[(int64_t)min(n0 / kBlockN + b, NBk - 1) * p.ws_n + (int64_t)(kb_begin + it) * p.ws_k];
+        }
+    }
+    const float *wsl = (const float *)(lds + Cfg::kWsOff) + (wave >> 2) * steps;
+
+    v4f acc[MT][TN];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    int slot = 0;
+    for (int it = 0; it < steps; ++it) {
+        // this wave's W rows and X groups of step `it` have landed; what was requested after them may be in flight:
+        // W(it+1), and with three slots X(it+1) and W(it+2)
+        if constexpr (NS == 2) {
+            if (it + 1 < steps) wait_vmcnt<4>();
+            else wait_vmcnt<0>();
+        } else {
+            if (it + 2 < steps) wait_vmcnt<8 + NXW>();
+            else if (it + 1 < steps) wait_vmcnt<4 + NXW>();
+            else wait_vmcnt<0>();
+        }
+        lds_barrier();  // step `it` is visible to all; everyone has finished reading step it - 1
+        {
+            const int xi = it + NS - 1;
+            if (xi < steps) {
+                issue_x(slot == 0 ? NS - 1 : slot - 1, xi);
+                if ((xi & 7) == 0) issue_scales(xi >> 3);
+            }
+        }
+        const uint8_t *st = lds + slot * Cfg::kStage;
+        const float ws_cur = wsl[it];
+        const float *sp = (const float *)(lds + sr8 + ((it >> 3) & 1) * Cfg::kChunkBytes + (it & 7) * 4);
+        v8i wf[TN], xf[MT];
+        float xs[MT];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
+            const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
+            wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
+            const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
+            xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            xs[i] = sp[i * 16 * 8] * ws_cur;
+        }
+        // the wave's own W rows of this slot have been read: request those of step it + NS into them
+        __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8));  // lgkmcnt(0)
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        if (it + NS < steps) issue_w(slot, it + NS);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const v4f part = mfma_16x16x128_fp8(wf[j], xf[i], v4f{0.f, 0.f, 0.f, 0.f});
+                acc[i][j] += part * xs[i];
+            }
+        slot = slot + 1 == NS ? 0 : slot + 1;
+    }
+
+    // ---- shared K range: the partial sums go to the workspace in register order ([wave][block][lane] float4);
+    // rows128_reduce_kernel adds them in split order and writes C
+    if constexpr (SPLIT) {
+        constexpr int F = MT * TN;
+        float *part = p.partials + ((int64_t)tile_n * p.splits + split) * Cfg::kTileElems + (wave * F * 64 + lane) * 4;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) *(v4f *)(part + (i * TN + j) * 256) = acc[i][j];
+        return;
+    }
+
+    // ---- epilogue: lane (r16, g4) holds row 16*i + r16 and the 8 columns n0 + 32*wave + 8*g4 + [0, 8)
+    const int nbase = n0 + wave * WNS;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int rl = 16 * i + r16;
+        if (rl >= p.M) continue;
+        uint16_t *cp = p.C + (int64_t)rl * p.ldc + nbase;
+        float o[4 * TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = acc[i][j][vv];
+        if (p.vec_store && nbase + WNS <= p.N) {
+            *(v4i *)(cp + lane_col<TN>(g4, 0)) =
+                v4i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16),
+                    (int)pack_out2(o[4], o[5], p.out_f16), (int)pack_out2(o[6], o[7], p.out_f16)};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4 * TN; ++e) {
+                const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
+                if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
+            }
+        }
+    }
+}
+
+// Second launch of a shared-K GEMM: thread (tile, wave, row block i, lane) adds its two accumulator blocks over the
+// splits in split order and stores 8 consecutive outputs of row 16*i + lane % 16.
+template <int MT>
+__global__ __launch_bounds__(256) void rows128_reduce_kernel(const GemmArgs p) {
+    using Cfg = Rows128Cfg<MT, 2>;
+    constexpr int TN = Cfg::TN, WNS = Cfg::WNS, F = MT * TN;
+    const int lane = threadIdx.x & 63;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);  // (tile, wave, i)
+    const int tiles = (p.N + Cfg::BN - 1) / Cfg::BN;
+    if (item >= tiles * Cfg::kWaves * MT) return;
+    const int i = item % MT, wave = (item / MT) % Cfg::kWaves, tile_n = item / (MT * Cfg::kWaves);
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const float *src = p.partials + (int64_t)tile_n * p.splits * Cfg::kTileElems + (wave * F * 64 + lane) * 4 + (i * TN) * 256;
+    v4f a0 = *(const v4f *)src, a1 = *(const v4f *)(src + 256);
+    int sp = 1;
+    for (; sp + 4 <= p.splits; sp += 4) {
+        v4f b0[4], b1[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            b0[d] = *(const v4f *)(src + (int64_t)(sp + d) * Cfg::kTileElems);
+            b1[d] = *(const v4f *)(src + (int64_t)(sp + d) * Cfg::kTileElems + 256);
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            a0 += b0[d];
+            a1 += b1[d];
+        }
+    }
+    for (; sp < p.splits; ++sp) {
+        a0 += *(const v4f *)(src + (int64_t)sp * Cfg::kTileElems);
+        a1 += *(const v4f *)(src + (int64_t)sp * Cfg::kTileElems + 256);
+    }
+    const int rl = 16 * i + r16;
+    if (rl >= p.M) return;
+    const int nbase = tile_n * Cfg::BN + wave * WNS;
+    uint16_t *cp = p.C + (int64_t)rl * p.ldc + nbase;
+    const float o[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+    if (p.vec_store && nbase + WNS <= p.N) {
+        *(v4i *)(cp + lane_col<TN>(g4, 0)) =
+            v4i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16),
+                (int)pack_out2(o[4], o[5], p.out_f16), (int)pack_out2(o[6], o[7], p.out_f16)};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
+            if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
+        }
+    }
+}
+
+}  // namespace mi355

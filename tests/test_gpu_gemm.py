@@ -57,7 +57,7 @@ def _check_small(xq, xs, wq, ws, C):
     assert err <= 2 ** -7, err
 
 
-@pytest.mark.parametrize("variant", [None, "tile256", "tile256x128", "tile128", "skinny", "generic"])
+@pytest.mark.parametrize("variant", [None, "tile256", "tile256x128", "tile128", "skinny", "rows128", "generic"])
 @pytest.mark.parametrize("M,N,K", [(32, 512, 1024), (1, 256, 512), (64, 384, 2048), (17, 2112, 256)])
 def test_small_vs_oracle(hip, M, N, K, variant):
     print(f"gemm small M={M} N={N} K={K} variant={variant}", flush=True)
@@ -247,6 +247,64 @@ def test_shared_activation_stream_kernel(hip):
     assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), _run(xq, xs, wq, ws, "xshare").view(torch.int16))
 
 
+def test_rows128_stream_kernel(hip):
+    """The 256-weight-row stream with the activation block in LDS (M <= 128): random shapes - every row-block
+    count, N tails that cut a wave's 32 rows, a workgroup's 256 rows and the vector stores, K from one step (fewer
+    steps than ring slots) to 144 so that whole-K and shared-K launches (second launch adds the partial sums) both
+    occur - against the torch fp32 dequant-matmul, the float64 oracle on a sample and the 128x128 tile (same
+    products in the same order when neither shares K: bit-equal); twice in a row (no state is left behind)."""
+    from lightllm_amd import _lib
+
+    rng = np.random.default_rng(2718)
+    cases = [(int(rng.integers(1, 129)), int(rng.integers(1, 300)) * int(rng.choice([1, 8, 16, 32, 128])),
+              int(rng.choice([128, 256, 384, 640, 1024, 2048, 4096, 7168, 18432]))) for _ in range(20)]
+    cases += [(128, 256, 128), (65, 4096, 14336), (127, 2112, 7168), (80, 520, 2304)]
+    shared = 0
+    for case, (M, N, K) in enumerate(cases):
+        print(f"gemm rows128 case {case}: M={M} N={N} K={K}", flush=True)
+        xq, xs, wq, ws = _prep(M, N, K, seed=6000 + case, device="cuda")
+        c = _run(xq, xs, wq, ws, "rows128").clone()
+        assert not torch.isnan(c.float()).any()
+        assert torch.equal(c, _run(xq, xs, wq, ws, "rows128"))
+        ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+        cos, rel = H.gemm_metrics(c.float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (M, N, K, cos, rel)
+        t = _run(xq, xs, wq, ws, "tile128")
+        split_here = _lib.lib().mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_ROWS128) > 0
+        split_there = _lib.lib().mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_TILE128) > 0
+        shared += split_here
+        if not split_here and not split_there:
+            assert torch.equal(c.view(torch.int16), t.view(torch.int16)), (M, N, K)
+        else:
+            assert (c.float() - t.float()).abs().max() <= ref.abs().max() * 2 ** -7, (M, N, K)
+        rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 4)])
+        cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 30)])
+        ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                              ws.cpu().numpy(), np.arange(len(rows)), cols)
+        got = c[rows][:, cols].float().cpu().double().numpy()
+        assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
+    assert 4 <= shared <= len(cases) - 4, "both launch kinds must occur"
+
+
+def test_rows128_column_major_scales(hip):
+    print("gemm rows128 column-major scales", flush=True)
+    xq, xs, wq, ws = _prep(100, 512, 2048, seed=78)
+    xs_cm = xs.t().contiguous().t()
+    C = _run(xq, xs_cm, wq, ws, "rows128")
+    _check_small(xq, xs, wq, ws, C)
+    assert torch.equal(C, _run(xq, xs, wq, ws, "rows128"))
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
+                                   (128, 2112, 7168)])
+def test_rows128_where_the_table_sends_it(hip, M, N, K):
+    """Model linears with 33..128 rows that the shape table gives to the 256-weight-row stream."""
+    print(f"gemm rows128 table shape M={M} N={N} K={K}", flush=True)
+    _check_full(M, N, K, None, seed=M + N % 89)
+    xq, xs, wq, ws = _prep(M, N, K, seed=1)
+    assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), _run(xq, xs, wq, ws, "rows128").view(torch.int16))
+
+
 def test_unit_scales_is_plain_matmul(hip):
     """All scales 1: the result is the plain product of the fp8 values, exact in fp32 for K=128."""
     print("gemm unit scales", flush=True)
@@ -256,7 +314,7 @@ def test_unit_scales_is_plain_matmul(hip):
     b = torch.randint(-8, 9, (N, K), generator=g).float().to(torch.float8_e4m3fn).cuda()
     ones_a = torch.ones((M, 1), dtype=torch.float32, device="cuda")
     ones_b = torch.ones((2, 1), dtype=torch.float32, device="cuda")
-    for variant in [None, "tile128", "tile256", "skinny", "generic"]:
+    for variant in [None, "tile128", "tile256", "skinny", "rows128", "generic"]:
         C = _run(a, ones_a, b, ones_b, variant)
         ref = (a.float().cpu().double() @ b.float().cpu().double().T)
         # integers up to 128*64 = 8192 need 13 bits; bf16 keeps 8: compare after the same rounding
@@ -274,7 +332,7 @@ def test_one_hot_rows_pick_scaled_columns(hip):
     a[torch.arange(M), ks] = 1.0
     aq = a.to(torch.float8_e4m3fn).cuda()
     As = (torch.rand((M, K // 128), generator=g) + 0.5).cuda()
-    for variant in [None, "tile128", "skinny"]:
+    for variant in [None, "tile128", "skinny", "rows128"]:
         C = _run(aq, As, wq, ws, variant)
         kb = (ks // 128).cuda()
         sa = As[torch.arange(M, device="cuda"), kb]                       # [M]
@@ -288,12 +346,15 @@ def test_one_hot_rows_pick_scaled_columns(hip):
 
 @pytest.mark.parametrize("M,N,K", [(128, 512, 4096), (200, 640, 8192), (65, 256, 2048)])
 def test_mid_m_split_k_tiles(hip, M, N, K):
-    """Few 128x128 tiles and a long K: the tiled kernel shares the K range between CTAs."""
+    """Few 128x128 tiles and a long K: the tiled kernel shares the K range between CTAs.  (The shape table sends
+    at most 128 rows with K >= 2048 to the 256-weight-row stream instead.)"""
     print(f"gemm mid-M split-K M={M} N={N} K={K}", flush=True)
     xq, xs, wq, ws = _prep(M, N, K, seed=M + K)
     C1 = _run(xq, xs, wq, ws, None).clone()
     C2 = _run(xq, xs, wq, ws, "tile128").clone()
-    assert torch.equal(C1, C2) and torch.equal(C2, _run(xq, xs, wq, ws, "tile128"))
+    assert torch.equal(C1, _run(xq, xs, wq, ws, "rows128" if M <= 128 else "tile128"))
+    assert torch.equal(C2, _run(xq, xs, wq, ws, "tile128"))
+    assert (C1.float() - C2.float()).abs().max() <= C2.float().abs().max() * 2 ** -7
     ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
     cos, rel = H.gemm_metrics(C1.float(), ref)
     assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
@@ -427,6 +488,7 @@ def test_quant_method_apply(hip):
 @pytest.mark.parametrize("variant,M,N,K", [("tile256", 300, 1000, 1152), ("tile256once", 512, 512, 1024), ("tile128", 130, 520, 512),
                                            ("tile256x128", 260, 300, 256), ("skinny", 9, 1000, 2048), ("skinny", 40, 4100, 4096),
                                            ("xshare", 50, 4096, 1024), ("tile256streamk", 1000, 2048, 16384),
+                                           ("rows128", 100, 1000, 512), ("rows128", 128, 4104, 14336),
                                            ("generic", 7, 130, 256), (None, 64, 28672, 4096), (None, 1024, 2112, 7168)])
 def test_fp16_output(hip, variant, M, N, K):
     """C in fp16: the fp32 accumulator is cast to the dtype of C (fp8w8a8_block_gemm_kernel.py:78; LightLLM allocates C
