@@ -277,7 +277,7 @@ def main():
             ncopies = -(-640_000_000 // (Nd * Kd))
             copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(ncopies)]
             views = [(q.t(), s.t()) for q, s in copies]
-            for Md in (1, 8, 32, 64):
+            for Md in (1, 8, 32, 64, 128):
                 xq, xs = per_token_group_quant_fp8(make_act(Md, Kd, 20 + Md, dev), 128)
                 out = torch.empty((Md, Nd), dtype=torch.bfloat16, device=dev)
                 nxt = _rotating(views)

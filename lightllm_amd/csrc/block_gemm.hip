@@ -206,6 +206,11 @@ static SkinnyPlan skinny_plan(int64_t M, int64_t N, int64_t K, int cus) {
     const int max_splits = KB / 16 > 0 ? KB / 16 : 1;
     if (pl.splits > max_splits) pl.splits = max_splits;
     if (pl.splits < 1) pl.splits = 1;
+    // a workgroup stages the activation scales of its K range in LDS if the range is short enough; one more split
+    // that gets it there pays (N=7168, K=18432, M=16: 72 steps unstaged 37.5 us, 48 steps staged 30.7)
+    const int cap = skinny_mt(M) == 4 ? StreamCfg<4, 2>::kMaxScaleSteps : StreamCfg<1, 1>::kMaxScaleSteps;
+    const int need = (KB + cap - 1) / cap;
+    if (pl.splits < need && need <= max_splits) pl.splits = need;
     return pl;
 }
 

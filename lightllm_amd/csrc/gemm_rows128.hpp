@@ -5,7 +5,7 @@
 // is bound by the latency of its steps, not by the memory.  This kernel is the 64-row tile of the grouped GEMM
 // (gemm_small.hpp) with twice the rows and a dense epilogue:
 //
-//   16*MT activation rows (MT = 5..8 MFMA row blocks) x 256 weight rows, K step 128.
+//   16*MT activation rows (MT = 1..8 MFMA row blocks) x 256 weight rows, K step 128.
 //   8 waves, wave w owns weight rows [32w, 32w+32) and all activation rows: MT x 2 MFMA blocks per K step.
 //   NS ring slots of { X 16*MT x 128 B, W 256 x 128 B }.  A wave fetches its own W rows (4 requests of 1 KiB per
 //   step) into its own part of a slot and is the only one to read them, so the W stream needs no barrier: the rows
@@ -13,9 +13,14 @@
 //   per step makes step kb visible and frees the slot of step kb - 1 for step kb + NS - 1.
 //   X scales come in [rows][8 steps] chunks by 4-byte requests (any scale layout); the W scales of the tile's two
 //   128-wide n blocks are copied to LDS once.
-//   When N / 256 tiles are too few for the device the K range is shared between workgroups.  Their partial sums
+//   A compute unit pulls 35 to 40 GB/s from HBM through this tile, so the launch wants a workgroup on every unit:
+//   when the N / 256 tiles are too few for that the K range is shared between workgroups.  Their partial sums
 //   are 16*MT x 256 floats each, too many for the last workgroup of a tile to add alone (one compute unit reads
 //   about 40 GB/s): they go to the workspace and a second, device-wide launch adds them in split order.
+//
+//   (Half-width tiles of four waves on two slots, two workgroups to a unit, were tried for shapes whose 256-row
+//   tiles leave units idle and cannot share K usefully - N = 36864: 144 tiles on 256 units - and were slower: 85 us
+//   against 69 at M = 128.)
 //
 // Arithmetic, operand layouts in LDS and the epilogue are those of the other tiled kernels (gemm_tile.hpp).
 #pragma once
@@ -177,6 +182,11 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
             const v4i hi = *(const v4i *)(st + wr1 + j * 2048);
             wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         }
+        // the wave's own W rows of this slot have been read: request those of step it + NS into them.  (Only the
+        // W reads are waited for here; the X reads below overlap the products.)
+        __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8));  // lgkmcnt(0)
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);
+        if (it + NS < steps) issue_w(slot, it + NS);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
@@ -184,10 +194,6 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
             xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             xs[i] = sp[i * 16 * 8] * ws_cur;
         }
-        // the wave's own W rows of this slot have been read: request those of step it + NS into them
-        __builtin_amdgcn_s_waitcnt(0xf | (0x3 << 14) | (0x7 << 4) | (0 << 8));  // lgkmcnt(0)
-        __atomic_signal_fence(__ATOMIC_SEQ_CST);
-        if (it + NS < steps) issue_w(slot, it + NS);
 #pragma unroll
         for (int i = 0; i < MT; ++i)
 #pragma unroll
