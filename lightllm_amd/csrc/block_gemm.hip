@@ -314,70 +314,83 @@ static int launch_xshare(GemmArgs &a, int splits, void *ws, hipStream_t st) {
     return launch(kernel, dim3(tiles * splits), dim3(256), lds_bytes, st, a);
 }
 
-// ---- 65..128 rows: the weight stream with the activation block in LDS (gemm_rows128.hpp)
-#ifndef MI355_ROWS128_NS
-#define MI355_ROWS128_NS 3
-#endif
-constexpr int kRows128Slots = MI355_ROWS128_NS;
+// ---- at most 256 rows: the weight stream with the activation block in LDS (gemm_rows128.hpp).  Up to 128 rows a
+// workgroup takes 256 weight rows on three ring slots, beyond that 128 weight rows on two (the activation block of a
+// step is twice as large).
 constexpr int kRows128MinSteps = 6;
 
 static int rows128_mt(int64_t M) { return (int)((M + 15) / 16); }
+static int rows128_bn(int64_t M) { return M <= 128 ? 256 : 128; }
 
-// N / 256 workgroup tiles; while they leave compute units idle the K range is shared, never below kRows128MinSteps
+// N / BN workgroup tiles; while they leave compute units idle the K range is shared, never below kRows128MinSteps
 // K steps for a workgroup.
-static int rows128_splits(int64_t N, int64_t K, int cus) {
-    const int64_t tiles = (N + 255) / 256, KB = K / kBlockK;
+static int rows128_splits(int64_t M, int64_t N, int64_t K, int cus) {
+    const int bn = rows128_bn(M);
+    const int64_t tiles = (N + bn - 1) / bn, KB = K / kBlockK;
     int64_t splits = cus / tiles;
     if (splits > KB / kRows128MinSteps) splits = KB / kRows128MinSteps;
     return (int)(splits < 1 ? 1 : splits);
 }
 
 static size_t rows128_workspace(int64_t M, int64_t N, int splits) {
-    const int64_t tiles = (N + 255) / 256;
-    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 16 * rows128_mt(M) * 256 * 4;
+    const int bn = rows128_bn(M);
+    const int64_t tiles = (N + bn - 1) / bn;
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 16 * rows128_mt(M) * bn * 4;
 }
 
 // Where the kernel pays (Llama-3-8B and DeepSeek-V3 linears, weights rotated so that none is found in the
-// memory-side cache).  Above 64 rows it beats the 128x128 tiles by 10 to 30 % (DeepSeek-V3 down, M = 128: 39.5 us
+// memory-side cache).  At 65..128 rows it beats the 128x128 tiles by 10 to 30 % (DeepSeek-V3 down, M = 128: 39.5 us
 // against 50.0; Llama-3 down: 27.9 against 30.3) unless K is short (q_b, K = 1536: 21.7 against 17.0).  At 33..64
 // rows it beats the streaming kernels on the large weights (DeepSeek-V3 gate_up, down, o at M = 64: 58.4, 31.7,
 // 31.9 us against 72.3, 42.5, 43.1) and loses on the small ones, where its second launch shows (Llama-3 qkv: 15.0
 // against 13.1); at 32 rows and fewer the streaming kernels are the faster ones.
 static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
-    if (M <= 32 || M > 128) return false;
+    if (M <= 32 || M > 256) return false;
+    if (M > 128) {
+        // 129..256 rows, 128-row tiles.  Against the 128x128 tiles it wins where those are few and K is long
+        // (DeepSeek-V3 down at M = 129 / 256: 44.8 / 62.4 us against 83.9 / 84.6; Llama-3 down 25.3 / 34.7 against
+        // 42.5), and up to 160 rows also where the tiles about fill the device (Llama-3 gate_up, 224 tiles, M = 160:
+        // 40.1 against 46.7; M = 192: 49.2 against 46.8).  With more tiles than units it loses (DeepSeek-V3 gate_up).
+        const int64_t tiles = (N + 127) / 128;
+        if (K / kBlockK < 16) return false;
+        if (tiles * 2 <= cus) return tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
+        return M <= 160 && tiles <= cus;
+    }
     if (M > 64) return K / kBlockK >= 16;
     if (N * K < 100000000ll) return false;
-    return rows128_splits(N, K, cus) == 1 || !xshare_pays(M, N, K, cus);
+    return rows128_splits(M, N, K, cus) == 1 || !xshare_pays(M, N, K, cus);
 }
 
 static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t as_m, int64_t as_k, int cus) {
-    if (M > 128) return false;
+    if (M > 256) return false;
     if (M * lda >= (1ll << 32) || M * as_m * 4 >= (1ll << 32) || as_k * 32 >= (1ll << 32)) return false;
-    const int splits = rows128_splits(N, K, cus);
+    const int splits = rows128_splits(M, N, K, cus);
     const int64_t steps = (K / kBlockK + splits - 1) / splits;
-    return Rows128Cfg<8, kRows128Slots>::lds_bytes((int)steps) <= 160 * 1024;
+    if (M > 128) return Rows128Cfg<16, 2, 1>::lds_bytes((int)steps) <= 160 * 1024;
+    return Rows128Cfg<8, 3, 2>::lds_bytes((int)steps) <= 160 * 1024;
 }
 
 template <int MT>
 static int launch_rows128(GemmArgs &a, int splits, void *ws, hipStream_t st) {
-    using Cfg = Rows128Cfg<MT, kRows128Slots>;
+    constexpr int TN = MT <= 8 ? 2 : 1, NS = MT <= 8 ? 3 : 2;
+    using Cfg = Rows128Cfg<MT, NS, TN>;
     const int KB = a.K / kBlockK;
     const int steps = (KB + splits - 1) / splits;
     const int lds_bytes = Cfg::lds_bytes(steps);
     if (lds_bytes > 160 * 1024) return MI355_EUNSUPPORTED;
     const int tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
     if (splits <= 1) {
-        constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, kRows128Slots, false>;
+        constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, false>;
         if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
         return launch(kernel, dim3(tiles), dim3(Cfg::kThreads), lds_bytes, st, a);
     }
-    constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, kRows128Slots, true>;
+    constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, true>;
     if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
     a.splits = splits;
     a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);  // the counter words stay untouched
     const int r = launch(kernel, dim3(tiles * splits), dim3(Cfg::kThreads), lds_bytes, st, a);
     if (r != MI355_OK) return r;
-    return launch(rows128_reduce_kernel<MT>, dim3((tiles * Cfg::kWaves * MT + 3) / 4), dim3(256), 0, st, a);
+    return launch(rows128_reduce_kernel<MT, TN>, dim3((tiles * Cfg::kWaves * MT + 3) / 4), dim3(256), 0, st, a);
 }
 
 static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n) {
@@ -386,7 +399,9 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 }
 
 // The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
-//   65 <= M <= 128, K >= 2048                        the 256-weight-row stream with the activation block in LDS
+//   129 <= M <= 256, K >= 2048, at most cus/2 tiles
+//     of 128 weight rows (cus if M <= 160)           the weight stream with the activation block in LDS
+//   65 <= M <= 128, K >= 2048                        the same with 256 weight rows per workgroup
 //   33 <= M <= 64, N*K >= 1e8                        the same, unless it would have to share K between workgroups
 //                                                    where the kernel below runs (Llama-3 gate_up: 30.7 us against 29.8)
 //   M <= 64                                          weight streaming (M > 32 and N/128 about the unit count: the
@@ -448,8 +463,8 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
         return splits > 1 ? xshare_workspace(N, splits) : 0;
     }
     if (variant == MI355_GEMM_ROWS128) {
-        if (M > 128) return 0;
-        const int splits = rows128_splits(N, K, cus);
+        if (M > 256) return 0;
+        const int splits = rows128_splits(M, N, K, cus);
         return splits > 1 ? rows128_workspace(M, N, splits) : 0;
     }
     if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
@@ -493,8 +508,8 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
         // the table's other choice where a limit of the 256-row stream is not met or its partial sums have no room
         if (variant == MI355_GEMM_ROWS128 &&
             (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus) ||
-             (rows128_splits(N, K, cus) > 1 &&
-              (!ws || ws_bytes < rows128_workspace(M, N, rows128_splits(N, K, cus)) || ((uintptr_t)ws & 15)))))
+             (rows128_splits(M, N, K, cus) > 1 &&
+              (!ws || ws_bytes < rows128_workspace(M, N, rows128_splits(M, N, K, cus)) || ((uintptr_t)ws & 15)))))
             variant = pick_variant(M, N, K, cus, false);
         if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
             variant = MI355_GEMM_TILE128;
@@ -573,7 +588,7 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
         }
         case MI355_GEMM_ROWS128: {
             if (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus)) return MI355_EUNSUPPORTED;
-            const int splits = rows128_splits(N, K, cus);
+            const int splits = rows128_splits(M, N, K, cus);
             if (splits > 1 && (!ws || ws_bytes < rows128_workspace(M, N, splits) || ((uintptr_t)ws & 15)))
                 return MI355_EWORKSPACE;
             switch (rows128_mt(M)) {
@@ -584,7 +599,15 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
                 case 5: return launch_rows128<5>(a, splits, ws, st);
                 case 6: return launch_rows128<6>(a, splits, ws, st);
                 case 7: return launch_rows128<7>(a, splits, ws, st);
-                default: return launch_rows128<8>(a, splits, ws, st);
+                case 8: return launch_rows128<8>(a, splits, ws, st);
+                case 9: return launch_rows128<9>(a, splits, ws, st);
+                case 10: return launch_rows128<10>(a, splits, ws, st);
+                case 11: return launch_rows128<11>(a, splits, ws, st);
+                case 12: return launch_rows128<12>(a, splits, ws, st);
+                case 13: return launch_rows128<13>(a, splits, ws, st);
+                case 14: return launch_rows128<14>(a, splits, ws, st);
+                case 15: return launch_rows128<15>(a, splits, ws, st);
+                default: return launch_rows128<16>(a, splits, ws, st);
             }
         }
         case MI355_GEMM_SKINNY: {

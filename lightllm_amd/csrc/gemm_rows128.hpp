@@ -28,25 +28,46 @@
 
 namespace mi355 {
 
-template <int MT, int NS>
+template <int MT, int NS, int TN_ = 2>
 struct Rows128Cfg {
-    static_assert(MT >= 1 && MT <= 8 && (NS == 2 || NS == 3), "");
-    static constexpr int BN = 256, kWaves = 8, kThreads = 512, TN = 2, WNS = 32;
+    static_assert(MT >= 1 && MT <= 16 / TN_ && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
+    static constexpr int TN = TN_, WNS = 16 * TN, kWaves = 8, kThreads = 512, BN = WNS * kWaves;
+    static constexpr int NBLK = (BN + kBlockN - 1) / kBlockN;  // 128-wide n blocks of a tile
+    static constexpr int NWW = 2 * TN;                         // W requests per wave and step (8 rows each)
     static constexpr int XG = 2 * MT;                          // 8-row request groups of the X block
     static constexpr int NXW = (XG + kWaves - 1) / kWaves;     // X requests per wave (groups repeat if XG % 8 != 0)
+    static constexpr int XH = MT < 8 ? MT : 8;                 // X row blocks read from LDS at a time
     static constexpr int kXBytes = 16 * MT * 128, kWBytes = BN * 128;
     static constexpr int kStage = kXBytes + kWBytes;
-    static constexpr int kWsOff = NS * kStage;                 // W scales [2 n blocks][steps]
+    static constexpr int kWsOff = NS * kStage;                 // W scales [NBLK][steps]
     static constexpr int kChunkBytes = 16 * MT * 32;           // one [rows][8 steps] chunk of X scales
     static constexpr int kTileElems = 16 * MT * BN;
-    static constexpr int chunk_off(int steps) { return (kWsOff + 2 * steps * 4 + 127) & ~127; }
+    static constexpr int chunk_off(int steps) { return (kWsOff + NBLK * steps * 4 + 127) & ~127; }
     static constexpr int lds_bytes(int steps) { return chunk_off(steps) + 2 * kChunkBytes; }
 };
 
-template <int MT, int NS, bool SPLIT>
+// One lane's 4*TN consecutive outputs of row `row`: columns nbase + 4*TN*g4 + [0, 4*TN).
+template <int TN>
+__device__ __forceinline__ void rows128_store(const GemmArgs &p, int row, int nbase, int g4, const float *o) {
+    uint16_t *cp = p.C + (int64_t)row * p.ldc + nbase + lane_col<TN>(g4, 0);
+    if (p.vec_store && nbase + 16 * TN <= p.N) {
+        if constexpr (TN == 2) {
+            *(v4i *)cp = v4i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16),
+                             (int)pack_out2(o[4], o[5], p.out_f16), (int)pack_out2(o[6], o[7], p.out_f16)};
+        } else {
+            *(v2i *)cp = v2i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16)};
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4 * TN; ++e)
+            if (nbase + lane_col<TN>(g4, 0) + e < p.N) cp[e] = (uint16_t)out_bits(o[e], p.out_f16);
+    }
+}
+
+template <int MT, int NS, int TN, bool SPLIT>
 __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmArgs p) {
-    using Cfg = Rows128Cfg<MT, NS>;
-    constexpr int TN = Cfg::TN, WNS = Cfg::WNS, NXW = Cfg::NXW, XG = Cfg::XG;
+    using Cfg = Rows128Cfg<MT, NS, TN>;
+    constexpr int WNS = Cfg::WNS, NXW = Cfg::NXW, XG = Cfg::XG, NWW = Cfg::NWW, XH = Cfg::XH;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -84,10 +105,10 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         sc_row[i] = src * (uint32_t)p.xs_m;
         sdst[i] = (uint32_t)g * 256u;
     }
-    uint32_t woff[4];
+    uint32_t woff[NWW];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int w = 8 * i + sub;  // LDS row inside the wave's 32-row span
+    for (int i = 0; i < NWW; ++i) {
+        const int w = 8 * i + sub;  // LDS row inside the wave's span of 16*TN rows
         const int tn = w >> 4, gg = (w >> 2) & 3, vv = w & 3;
         const int nl = wave * WNS + lane_col<TN>(gg, tn) + vv;
         const int nc = min(n0 + nl, p.N - 1) - n0;
@@ -102,7 +123,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         const uint32_t sb = lds0 + (uint32_t)slot * Cfg::kStage + wdst;
         const uint8_t *wk = wg + (int64_t)it * kBlockK;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma_g2l_b128(sb + (uint32_t)i * 1024u, wk, woff[i]);
+        for (int i = 0; i < NWW; ++i) dma_g2l_b128(sb + (uint32_t)i * 1024u, wk, woff[i]);
     };
     auto issue_x = [&](int slot, int it) {
         const uint32_t sb = lds0 + (uint32_t)slot * Cfg::kStage;
@@ -138,12 +159,12 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
     {
         const int NBk = (p.N + kBlockN - 1) / kBlockN;
         float *wl = (float *)(lds + Cfg::kWsOff);
-        for (int i = tid; i < 2 * steps; i += Cfg::kThreads) {
+        for (int i = tid; i < Cfg::NBLK * steps; i += Cfg::kThreads) {
             const int b = i >= steps ? 1 : 0, it = i - b * steps;
             wl[i] = p.Ws[(int64_t)min(n0 / kBlockN + b, NBk - 1) * p.ws_n + (int64_t)(kb_begin + it) * p.ws_k];
         }
     }
-    const float *wsl = (const float *)(lds + Cfg::kWsOff) + (wave >> 2) * steps;
+    const float *wsl = (const float *)(lds + Cfg::kWsOff) + ((wave * WNS) / kBlockN) * steps;
 
     v4f acc[MT][TN];
 #pragma unroll
@@ -156,11 +177,11 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         // this wave's W rows and X groups of step `it` have landed; what was requested after them may be in flight:
         // W(it+1), and with three slots X(it+1) and W(it+2)
         if constexpr (NS == 2) {
-            if (it + 1 < steps) wait_vmcnt<4>();
+            if (it + 1 < steps) wait_vmcnt<NWW>();
             else wait_vmcnt<0>();
         } else {
-            if (it + 2 < steps) wait_vmcnt<8 + NXW>();
-            else if (it + 1 < steps) wait_vmcnt<4 + NXW>();
+            if (it + 2 < steps) wait_vmcnt<2 * NWW + NXW>();
+            else if (it + 1 < steps) wait_vmcnt<NWW + NXW>();
             else wait_vmcnt<0>();
         }
         lds_barrier();  // step `it` is visible to all; everyone has finished reading step it - 1
@@ -174,8 +195,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         const uint8_t *st = lds + slot * Cfg::kStage;
         const float ws_cur = wsl[it];
         const float *sp = (const float *)(lds + sr8 + ((it >> 3) & 1) * Cfg::kChunkBytes + (it & 7) * 4);
-        v8i wf[TN], xf[MT];
-        float xs[MT];
+        v8i wf[TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
             const v4i lo = *(const v4i *)(st + wr0 + j * 2048);
@@ -188,19 +208,27 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         if (it + NS < steps) issue_w(slot, it + NS);
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const v4i lo = *(const v4i *)(st + xr0 + i * 2048);
-            const v4i hi = *(const v4i *)(st + xr1 + i * 2048);
-            xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            xs[i] = sp[i * 16 * 8] * ws_cur;
+        for (int h = 0; h < MT; h += XH) {  // at most 8 row blocks of X in registers at a time
+            v8i xf[XH];
+            float xs[XH];
+#pragma unroll
+            for (int i = 0; i < XH; ++i)
+                if (h + i < MT) {
+                    const v4i lo = *(const v4i *)(st + xr0 + (h + i) * 2048);
+                    const v4i hi = *(const v4i *)(st + xr1 + (h + i) * 2048);
+                    xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    xs[i] = sp[(h + i) * 16 * 8] * ws_cur;
+                }
+#pragma unroll
+            for (int i = 0; i < XH; ++i)
+                if (h + i < MT) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        const v4f part = mfma_16x16x128_fp8(wf[j], xf[i], v4f{0.f, 0.f, 0.f, 0.f});
+                        acc[h + i][j] += part * xs[i];
+                    }
+                }
         }
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const v4f part = mfma_16x16x128_fp8(wf[j], xf[i], v4f{0.f, 0.f, 0.f, 0.f});
-                acc[i][j] += part * xs[i];
-            }
         slot = slot + 1 == NS ? 0 : slot + 1;
     }
 
@@ -216,38 +244,27 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         return;
     }
 
-    // ---- epilogue: lane (r16, g4) holds row 16*i + r16 and the 8 columns n0 + 32*wave + 8*g4 + [0, 8)
+    // ---- epilogue: lane (r16, g4) holds row 16*i + r16 and the 4*TN columns n0 + 16*TN*wave + 4*TN*g4 + [0, 4*TN)
     const int nbase = n0 + wave * WNS;
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int rl = 16 * i + r16;
         if (rl >= p.M) continue;
-        uint16_t *cp = p.C + (int64_t)rl * p.ldc + nbase;
         float o[4 * TN];
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = acc[i][j][vv];
-        if (p.vec_store && nbase + WNS <= p.N) {
-            *(v4i *)(cp + lane_col<TN>(g4, 0)) =
-                v4i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16),
-                    (int)pack_out2(o[4], o[5], p.out_f16), (int)pack_out2(o[6], o[7], p.out_f16)};
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4 * TN; ++e) {
-                const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
-                if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
-            }
-        }
+        rows128_store<TN>(p, rl, nbase, g4, o);
     }
 }
 
-// Second launch of a shared-K GEMM: thread (tile, wave, row block i, lane) adds its two accumulator blocks over the
-// splits in split order and stores 8 consecutive outputs of row 16*i + lane % 16.
-template <int MT>
+// Second launch of a shared-K GEMM: thread (tile, wave, row block i, lane) adds its TN accumulator blocks over the
+// splits in split order and stores 4*TN consecutive outputs of row 16*i + lane % 16.
+template <int MT, int TN>
 __global__ __launch_bounds__(256) void rows128_reduce_kernel(const GemmArgs p) {
-    using Cfg = Rows128Cfg<MT, 2>;
-    constexpr int TN = Cfg::TN, WNS = Cfg::WNS, F = MT * TN;
+    using Cfg = Rows128Cfg<MT, 2, TN>;
+    constexpr int WNS = Cfg::WNS, F = MT * TN;
     const int lane = threadIdx.x & 63;
     const int item = blockIdx.x * 4 + (threadIdx.x >> 6);  // (tile, wave, i)
     const int tiles = (p.N + Cfg::BN - 1) / Cfg::BN;
@@ -255,41 +272,32 @@ __global__ __launch_bounds__(256) void rows128_reduce_kernel(const GemmArgs p) {
     const int i = item % MT, wave = (item / MT) % Cfg::kWaves, tile_n = item / (MT * Cfg::kWaves);
     const int r16 = lane & 15, g4 = lane >> 4;
     const float *src = p.partials + (int64_t)tile_n * p.splits * Cfg::kTileElems + (wave * F * 64 + lane) * 4 + (i * TN) * 256;
-    v4f a0 = *(const v4f *)src, a1 = *(const v4f *)(src + 256);
+    v4f a[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) a[j] = *(const v4f *)(src + j * 256);
     int sp = 1;
     for (; sp + 4 <= p.splits; sp += 4) {
-        v4f b0[4], b1[4];
+        v4f b[4][TN];
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            b0[d] = *(const v4f *)(src + (int64_t)(sp + d) * Cfg::kTileElems);
-            b1[d] = *(const v4f *)(src + (int64_t)(sp + d) * Cfg::kTileElems + 256);
-        }
+        for (int d = 0; d < 4; ++d)
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            a0 += b0[d];
-            a1 += b1[d];
-        }
+            for (int j = 0; j < TN; ++j) b[d][j] = *(const v4f *)(src + (int64_t)(sp + d) * Cfg::kTileElems + j * 256);
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) a[j] += b[d][j];
     }
-    for (; sp < p.splits; ++sp) {
-        a0 += *(const v4f *)(src + (int64_t)sp * Cfg::kTileElems);
-        a1 += *(const v4f *)(src + (int64_t)sp * Cfg::kTileElems + 256);
-    }
+    for (; sp < p.splits; ++sp)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) a[j] += *(const v4f *)(src + (int64_t)sp * Cfg::kTileElems + j * 256);
     const int rl = 16 * i + r16;
     if (rl >= p.M) return;
-    const int nbase = tile_n * Cfg::BN + wave * WNS;
-    uint16_t *cp = p.C + (int64_t)rl * p.ldc + nbase;
-    const float o[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-    if (p.vec_store && nbase + WNS <= p.N) {
-        *(v4i *)(cp + lane_col<TN>(g4, 0)) =
-            v4i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16),
-                (int)pack_out2(o[4], o[5], p.out_f16), (int)pack_out2(o[6], o[7], p.out_f16)};
-    } else {
+    float o[4 * TN];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
-            if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
-        }
-    }
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = a[j][vv];
+    rows128_store<TN>(p, rl, tile_n * Cfg::BN + wave * WNS, g4, o);
 }
 
 }  // namespace mi355

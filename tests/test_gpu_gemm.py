@@ -248,8 +248,9 @@ def test_shared_activation_stream_kernel(hip):
 
 
 def test_rows128_stream_kernel(hip):
-    """The 256-weight-row stream with the activation block in LDS (M <= 128): random shapes - every row-block
-    count, N tails that cut a wave's 32 rows, a workgroup's 256 rows and the vector stores, K from one step (fewer
+    """The weight stream with the activation block in LDS (M <= 256; 256 weight rows per workgroup up to 128 rows,
+    128 beyond): random shapes - every row-block
+    count, N tails that cut a wave's rows, a workgroup's rows and the vector stores, K from one step (fewer
     steps than ring slots) to 144 so that whole-K and shared-K launches (second launch adds the partial sums) both
     occur - against the torch fp32 dequant-matmul, the float64 oracle on a sample and the 128x128 tile (same
     products in the same order when neither shares K: bit-equal); twice in a row (no state is left behind)."""
@@ -258,7 +259,10 @@ def test_rows128_stream_kernel(hip):
     rng = np.random.default_rng(2718)
     cases = [(int(rng.integers(1, 129)), int(rng.integers(1, 300)) * int(rng.choice([1, 8, 16, 32, 128])),
               int(rng.choice([128, 256, 384, 640, 1024, 2048, 4096, 7168, 18432]))) for _ in range(20)]
-    cases += [(128, 256, 128), (65, 4096, 14336), (127, 2112, 7168), (80, 520, 2304)]
+    cases += [(int(rng.integers(129, 257)), int(rng.integers(1, 300)) * int(rng.choice([1, 4, 8, 16, 128])),
+               int(rng.choice([128, 256, 640, 1024, 2048, 7168, 18432]))) for _ in range(14)]
+    cases += [(128, 256, 128), (65, 4096, 14336), (127, 2112, 7168), (80, 520, 2304), (256, 128, 128), (129, 7168, 2048),
+              (255, 2112, 7168), (144, 1000, 4096)]
     shared = 0
     for case, (M, N, K) in enumerate(cases):
         print(f"gemm rows128 case {case}: M={M} N={N} K={K}", flush=True)
@@ -296,9 +300,11 @@ def test_rows128_column_major_scales(hip):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
-                                   (128, 2112, 7168)])
+                                   (128, 2112, 7168), (256, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
+                                   (200, 6144, 4096)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
-    """Model linears with 33..128 rows that the shape table gives to the 256-weight-row stream."""
+    """Model linears with 33..256 rows that the shape table gives to the weight stream with the activation block in
+    LDS."""
     print(f"gemm rows128 table shape M={M} N={N} K={K}", flush=True)
     _check_full(M, N, K, None, seed=M + N % 89)
     xq, xs, wq, ws = _prep(M, N, K, seed=1)
@@ -488,7 +494,7 @@ def test_quant_method_apply(hip):
 @pytest.mark.parametrize("variant,M,N,K", [("tile256", 300, 1000, 1152), ("tile256once", 512, 512, 1024), ("tile128", 130, 520, 512),
                                            ("tile256x128", 260, 300, 256), ("skinny", 9, 1000, 2048), ("skinny", 40, 4100, 4096),
                                            ("xshare", 50, 4096, 1024), ("tile256streamk", 1000, 2048, 16384),
-                                           ("rows128", 100, 1000, 512), ("rows128", 128, 4104, 14336),
+                                           ("rows128", 100, 1000, 512), ("rows128", 128, 4104, 14336), ("rows128", 250, 1004, 4096),
                                            ("generic", 7, 130, 256), (None, 64, 28672, 4096), (None, 1024, 2112, 7168)])
 def test_fp16_output(hip, variant, M, N, K):
     """C in fp16: the fp32 accumulator is cast to the dtype of C (fp8w8a8_block_gemm_kernel.py:78; LightLLM allocates C

@@ -23,7 +23,7 @@ def _replay_matches(fn_eager, make_graph_outputs, replays=4):
         assert torch.equal(again.view(torch.int16), expect.view(torch.int16))
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 12288, 1024), (8, 4096, 14336), (200, 640, 8192), (100, 4096, 14336)])
+@pytest.mark.parametrize("M,N,K", [(4096, 12288, 1024), (8, 4096, 14336), (200, 640, 8192), (100, 4096, 14336), (200, 4096, 14336)])
 def test_quant_and_gemm_under_graph_capture(hip, M, N, K):
     """Persistent 256x256 launch (768 tiles), split-K stream launch, split-K 128x128 launch, the 256-weight-row
     stream with its second launch that adds the partial sums."""
