@@ -1,21 +1,23 @@
-// Block-scaled FP8 GEMM for 65..128 activation rows on gfx950: a weight stream with the activation block in LDS.
+// Block-scaled FP8 GEMM for at most 256 activation rows on gfx950: a weight stream with the activation block in LDS.
 //
-// With at most 128 rows of X every weight byte is used once per launch, so the launch is a stream over W, and the
-// square tiles spend it badly: a 128x128 tile keeps 16 KiB of W per K step in flight and one round of such tiles
+// With so few rows of X every weight byte is used once (TN = 2) per launch, so the launch is a stream over W, and
+// the square tiles spend it badly: a 128x128 tile keeps 16 KiB of W per K step in flight and one round of such tiles
 // is bound by the latency of its steps, not by the memory.  This kernel is the 64-row tile of the grouped GEMM
-// (gemm_small.hpp) with twice the rows and a dense epilogue:
+// (gemm_small.hpp) with more rows and a dense epilogue:
 //
-//   16*MT activation rows (MT = 1..8 MFMA row blocks) x 256 weight rows, K step 128.
-//   8 waves, wave w owns weight rows [32w, 32w+32) and all activation rows: MT x 2 MFMA blocks per K step.
-//   NS ring slots of { X 16*MT x 128 B, W 256 x 128 B }.  A wave fetches its own W rows (4 requests of 1 KiB per
-//   step) into its own part of a slot and is the only one to read them, so the W stream needs no barrier: the rows
+//   16*MT activation rows (MT MFMA row blocks) x 128*TN weight rows, K step 128.
+//     TN = 2: up to 128 rows (MT <= 8) against 256 weight rows; TN = 1: up to 256 rows (MT <= 16) against 128.
+//   8 waves, wave w owns 16*TN weight rows and all activation rows: MT x TN MFMA blocks per K step (the X operand
+//   blocks are read from LDS eight at a time).
+//   NS ring slots of { X 16*MT x 128 B, W 128*TN x 128 B }.  A wave fetches its own W rows (2*TN requests of 1 KiB
+//   per step) into its own part of a slot and is the only one to read them, so the W stream needs no barrier: the rows
 //   of step kb + NS are requested as soon as the wave has read those of step kb.  The X block is shared: one barrier
 //   per step makes step kb visible and frees the slot of step kb - 1 for step kb + NS - 1.
-//   X scales come in [rows][8 steps] chunks by 4-byte requests (any scale layout); the W scales of the tile's two
+//   X scales come in [rows][8 steps] chunks by 4-byte requests (any scale layout); the W scales of the tile's
 //   128-wide n blocks are copied to LDS once.
 //   A compute unit pulls 35 to 40 GB/s from HBM through this tile, so the launch wants a workgroup on every unit:
-//   when the N / 256 tiles are too few for that the K range is shared between workgroups.  Their partial sums
-//   are 16*MT x 256 floats each, too many for the last workgroup of a tile to add alone (one compute unit reads
+//   when the tiles are too few for that the K range is shared between workgroups.  Their partial sums are
+//   16*MT x 128*TN floats each, too many for the last workgroup of a tile to add alone (one compute unit reads
 //   about 40 GB/s): they go to the workspace and a second, device-wide launch adds them in split order.
 //
 //   (Half-width tiles of four waves on two slots, two workgroups to a unit, were tried for shapes whose 256-row
