@@ -117,7 +117,7 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
                                         deterministic); falls back to MI355_GEMM_TILE256 where sharing gains nothing */
 
 #define MI355_GEMM_SKINNY_XSHARE 9 /* weight streaming, M <= 64, the activation block of a K step shared by the workgroup */
-#define MI355_GEMM_ROWS128 10 /* weight streaming, M <= 256, the activation block of a K step in LDS: 256 weight rows per
+#define MI355_GEMM_ROWS128 10 /* weight streaming, M <= 384, the activation block of a K step in LDS: 256 weight rows per
                                  workgroup up to 128 rows, 128 beyond; a second launch adds the partial sums when K is shared */
 
 #define MI355_WS_COUNTER_BYTES 65536

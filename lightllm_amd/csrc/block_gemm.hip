@@ -314,9 +314,9 @@ static int launch_xshare(GemmArgs &a, int splits, void *ws, hipStream_t st) {
     return launch(kernel, dim3(tiles * splits), dim3(256), lds_bytes, st, a);
 }
 
-// ---- at most 256 rows: the weight stream with the activation block in LDS (gemm_rows128.hpp).  Up to 128 rows a
+// ---- at most 384 rows: the weight stream with the activation block in LDS (gemm_rows128.hpp).  Up to 128 rows a
 // workgroup takes 256 weight rows on three ring slots, beyond that 128 weight rows on two (the activation block of a
-// step is twice as large).
+// step is two to three times as large).
 constexpr int kRows128MinSteps = 6;
 
 static int rows128_mt(int64_t M) { return (int)((M + 15) / 16); }
@@ -345,7 +345,16 @@ static size_t rows128_workspace(int64_t M, int64_t N, int splits) {
 // 31.9 us against 72.3, 42.5, 43.1) and loses on the small ones, where its second launch shows (Llama-3 qkv: 15.0
 // against 13.1); at 32 rows and fewer the streaming kernels are the faster ones.
 static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
-    if (M <= 32 || M > 256) return false;
+    if (M <= 32 || M > 384) return false;
+    if (M > 256) {
+        // 257..384 rows (the activation block of a step is 48 KiB): still ahead where the 128-row tiles are few, K is
+        // long and the weights are not small (Llama-3 down at M = 257 / 384: 38.0 / 46.8 us against 66.3 / 66.5;
+        // DeepSeek-V3 down 70.6 / 86.6 against 97.7 / 106.4; Llama-3 qkv 26.0 / 32.0 against 36.3); on 15 MB of
+        // weights (q_a+kv_a) it is not (24.1 against 23.5 at M = 320)
+        const int64_t tiles = (N + 127) / 128;
+        return K / kBlockK >= 16 && N * K >= 20000000ll && tiles * 2 <= cus &&
+               tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
+    }
     if (M > 128) {
         // 129..256 rows, 128-row tiles.  Against the 128x128 tiles it wins where those are few and K is long
         // (DeepSeek-V3 down at M = 129 / 256: 44.8 / 62.4 us against 83.9 / 84.6; Llama-3 down 25.3 / 34.7 against
@@ -362,10 +371,11 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
 }
 
 static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t as_m, int64_t as_k, int cus) {
-    if (M > 256) return false;
+    if (M > 384) return false;
     if (M * lda >= (1ll << 32) || M * as_m * 4 >= (1ll << 32) || as_k * 32 >= (1ll << 32)) return false;
     const int splits = rows128_splits(M, N, K, cus);
     const int64_t steps = (K / kBlockK + splits - 1) / splits;
+    if (M > 256) return Rows128Cfg<24, 2, 1>::lds_bytes((int)steps) <= 160 * 1024;
     if (M > 128) return Rows128Cfg<16, 2, 1>::lds_bytes((int)steps) <= 160 * 1024;
     return Rows128Cfg<8, 3, 2>::lds_bytes((int)steps) <= 160 * 1024;
 }
@@ -399,8 +409,9 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 }
 
 // The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
-//   129 <= M <= 256, K >= 2048, at most cus/2 tiles
-//     of 128 weight rows (cus if M <= 160)           the weight stream with the activation block in LDS
+//   129 <= M <= 384, K >= 2048, at most cus/2 tiles
+//     of 128 weight rows (cus if M <= 160; above
+//     256 rows only if N*K >= 2e7)                   the weight stream with the activation block in LDS
 //   65 <= M <= 128, K >= 2048                        the same with 256 weight rows per workgroup
 //   33 <= M <= 64, N*K >= 1e8                        the same, unless it would have to share K between workgroups
 //                                                    where the kernel below runs (Llama-3 gate_up: 30.7 us against 29.8)
@@ -463,7 +474,7 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
         return splits > 1 ? xshare_workspace(N, splits) : 0;
     }
     if (variant == MI355_GEMM_ROWS128) {
-        if (M > 256) return 0;
+        if (M > 384) return 0;
         const int splits = rows128_splits(M, N, K, cus);
         return splits > 1 ? rows128_workspace(M, N, splits) : 0;
     }
@@ -607,7 +618,15 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
                 case 13: return launch_rows128<13>(a, splits, ws, st);
                 case 14: return launch_rows128<14>(a, splits, ws, st);
                 case 15: return launch_rows128<15>(a, splits, ws, st);
-                default: return launch_rows128<16>(a, splits, ws, st);
+                case 16: return launch_rows128<16>(a, splits, ws, st);
+                case 17: return launch_rows128<17>(a, splits, ws, st);
+                case 18: return launch_rows128<18>(a, splits, ws, st);
+                case 19: return launch_rows128<19>(a, splits, ws, st);
+                case 20: return launch_rows128<20>(a, splits, ws, st);
+                case 21: return launch_rows128<21>(a, splits, ws, st);
+                case 22: return launch_rows128<22>(a, splits, ws, st);
+                case 23: return launch_rows128<23>(a, splits, ws, st);
+                default: return launch_rows128<24>(a, splits, ws, st);
             }
         }
         case MI355_GEMM_SKINNY: {

@@ -1,4 +1,4 @@
-// Block-scaled FP8 GEMM for at most 256 activation rows on gfx950: a weight stream with the activation block in LDS.
+// Block-scaled FP8 GEMM for at most 384 activation rows on gfx950: a weight stream with the activation block in LDS.
 //
 // With so few rows of X every weight byte is used once (TN = 2) per launch, so the launch is a stream over W, and
 // the square tiles spend it badly: a 128x128 tile keeps 16 KiB of W per K step in flight and one round of such tiles
@@ -6,7 +6,7 @@
 // (gemm_small.hpp) with more rows and a dense epilogue:
 //
 //   16*MT activation rows (MT MFMA row blocks) x 128*TN weight rows, K step 128.
-//     TN = 2: up to 128 rows (MT <= 8) against 256 weight rows; TN = 1: up to 256 rows (MT <= 16) against 128.
+//     TN = 2: up to 128 rows (MT <= 8) against 256 weight rows; TN = 1: up to 384 rows (MT <= 24) against 128.
 //   8 waves, wave w owns 16*TN weight rows and all activation rows: MT x TN MFMA blocks per K step (the X operand
 //   blocks are read from LDS eight at a time).
 //   NS ring slots of { X 16*MT x 128 B, W 128*TN x 128 B }.  A wave fetches its own W rows (2*TN requests of 1 KiB
@@ -32,7 +32,7 @@ namespace mi355 {
 
 template <int MT, int NS, int TN_ = 2>
 struct Rows128Cfg {
-    static_assert(MT >= 1 && MT <= 16 / TN_ && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
+    static_assert(MT >= 1 && MT <= (TN_ == 2 ? 8 : 24) && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
     static constexpr int TN = TN_, WNS = 16 * TN, kWaves = 8, kThreads = 512, BN = WNS * kWaves;
     static constexpr int NBLK = (BN + kBlockN - 1) / kBlockN;  // 128-wide n blocks of a tile
     static constexpr int NWW = 2 * TN;                         // W requests per wave and step (8 rows each)

@@ -248,7 +248,7 @@ def test_shared_activation_stream_kernel(hip):
 
 
 def test_rows128_stream_kernel(hip):
-    """The weight stream with the activation block in LDS (M <= 256; 256 weight rows per workgroup up to 128 rows,
+    """The weight stream with the activation block in LDS (M <= 384; 256 weight rows per workgroup up to 128 rows,
     128 beyond): random shapes - every row-block
     count, N tails that cut a wave's rows, a workgroup's rows and the vector stores, K from one step (fewer
     steps than ring slots) to 144 so that whole-K and shared-K launches (second launch adds the partial sums) both
@@ -259,10 +259,10 @@ def test_rows128_stream_kernel(hip):
     rng = np.random.default_rng(2718)
     cases = [(int(rng.integers(1, 129)), int(rng.integers(1, 300)) * int(rng.choice([1, 8, 16, 32, 128])),
               int(rng.choice([128, 256, 384, 640, 1024, 2048, 4096, 7168, 18432]))) for _ in range(20)]
-    cases += [(int(rng.integers(129, 257)), int(rng.integers(1, 300)) * int(rng.choice([1, 4, 8, 16, 128])),
-               int(rng.choice([128, 256, 640, 1024, 2048, 7168, 18432]))) for _ in range(14)]
+    cases += [(int(rng.integers(129, 385)), int(rng.integers(1, 300)) * int(rng.choice([1, 4, 8, 16, 128])),
+               int(rng.choice([128, 256, 640, 1024, 2048, 7168, 18432]))) for _ in range(18)]
     cases += [(128, 256, 128), (65, 4096, 14336), (127, 2112, 7168), (80, 520, 2304), (256, 128, 128), (129, 7168, 2048),
-              (255, 2112, 7168), (144, 1000, 4096)]
+              (255, 2112, 7168), (144, 1000, 4096), (384, 640, 4096), (257, 136, 256), (383, 4100, 2048)]
     shared = 0
     for case, (M, N, K) in enumerate(cases):
         print(f"gemm rows128 case {case}: M={M} N={N} K={K}", flush=True)
@@ -301,9 +301,9 @@ def test_rows128_column_major_scales(hip):
 
 @pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
                                    (128, 2112, 7168), (256, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
-                                   (200, 6144, 4096)])
+                                   (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
-    """Model linears with 33..256 rows that the shape table gives to the weight stream with the activation block in
+    """Model linears with 33..384 rows that the shape table gives to the weight stream with the activation block in
     LDS."""
     print(f"gemm rows128 table shape M={M} N={N} K={K}", flush=True)
     _check_full(M, N, K, None, seed=M + N % 89)
