@@ -724,15 +724,20 @@ extern "C" int mi355_reset_workspace(void *ws, size_t ws_bytes, void *stream) {
 }
 
 extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts, int64_t N, int64_t K) {
-    (void)N;
+    (void)K;
     if (num_experts <= 0) return 64;
     const int64_t avg = num_pairs / num_experts;
+    // 256-row schedule blocks run as the persistent launch with two queues: blocks of more than 64 rows on the
+    // 256x256 ping-pong tile (it skips the empty 64-row halves of ragged blocks), the others on the 64x512
+    // weight-streaming tile.  That launch needs more tiles than compute units; where it has them it is the faster
+    // one from about 12 rows per expert on (256 experts, top-8, N=4096 K=7168: 512 tokens 1275 us against 1291 for
+    // 32-row blocks, 1024 tokens 1314 against 1500, 2048 tokens 1421 against 1885; the same within 1 % at 384
+    // tokens).  With fewer rows the 16-row tiles stream the weights at 6.0 TB/s and nothing beats them.
+    const bool two_queues = (int64_t)num_experts * ((N + 255) / 256) > device_cus();
+    if (avg > 64 || (two_queues && avg >= 12)) return 256;
     if (avg <= 16) return 16;
     if (avg <= 32) return 32;
-    if (avg <= 64) return 64;
-    // prefill-size batches: the 256x256 ping-pong tile (it skips the empty 64-row halves of ragged blocks)
-    (void)K;
-    return 256;
+    return 64;
 }
 
 extern "C" size_t mi355_grouped_workspace_bytes(int64_t table_rows) {

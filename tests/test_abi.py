@@ -48,6 +48,12 @@ def test_pure_host_entry_points():
     assert lib.mi355_grouped_block_m(32768, 256, 4096, 7168) == 256
     assert lib.mi355_grouped_block_m(32768, 256, 4096, 7168 + 128) == 256   # any K/128 takes the 256-row blocks
     assert lib.mi355_grouped_block_m(64, 256, 4096, 7168) == 16
+    # 12..64 rows per expert: the two-queue launch of 256-row blocks where it has more tiles than compute units
+    # (256 assumed without a device), the row-sized tiles otherwise
+    assert lib.mi355_grouped_block_m(8192, 256, 4096, 7168) == 256
+    assert lib.mi355_grouped_block_m(2048, 256, 4096, 7168) == 16
+    assert lib.mi355_grouped_block_m(8 * 24, 8, 4096, 7168) == 32
+    assert lib.mi355_grouped_block_m(8 * 50, 8, 4096, 7168) == 64
     assert lib.mi355_block_fp8_gemm_workspace_bytes(4096, 4096, 4096, 0) == 65536  # large M: tile counters only
     assert lib.mi355_block_fp8_gemm_workspace_bytes(8, 4096, 14336, 0) > 65536
 
