@@ -367,6 +367,9 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
     }
     if (M > 64) return K / kBlockK >= 16;
     if (N * K < 100000000ll) return false;
+    // more tiles than units (lm_head, N = 128256, K = 4096, M = 64: 116 us against 110 for the shared-activation
+    // streaming kernel, whose small workgroups fill the second round better)
+    if ((N + 255) / 256 > cus) return false;
     return rows128_splits(M, N, K, cus) == 1 || !xshare_pays(M, N, K, cus);
 }
 
