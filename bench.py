@@ -273,7 +273,7 @@ def main():
     if (run_all and not args.no_others) or args.only == "decode":
         # Llama-3-8B decode linears; the weights rotate through enough copies (> 600 MB) that no launch finds them
         # in the 256 MB memory-side cache
-        for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down")]:
+        for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down"), (128256, 4096, "lm_head")]:
             ncopies = -(-640_000_000 // (Nd * Kd))
             copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(ncopies)]
             views = [(q.t(), s.t()) for q, s in copies]
