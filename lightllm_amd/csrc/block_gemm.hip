@@ -320,22 +320,49 @@ static int launch_xshare(GemmArgs &a, int splits, void *ws, hipStream_t st) {
 constexpr int kRows128MinSteps = 6;
 
 static int rows128_mt(int64_t M) { return (int)((M + 15) / 16); }
-static int rows128_bn(int64_t M) { return M <= 128 ? 256 : 128; }
 
-// N / BN workgroup tiles; while they leave compute units idle the K range is shared, never below kRows128MinSteps
-// K steps for a workgroup.
-static int rows128_splits(int64_t M, int64_t N, int64_t K, int cus) {
-    const int bn = rows128_bn(M);
-    const int64_t tiles = (N + bn - 1) / bn, KB = K / kBlockK;
+// Workgroup width, K sharing and tile count of a launch.  Up to 128 rows a workgroup is 8 waves x 32 weight rows;
+// beyond, 8 waves x 16.  While the tiles leave compute units idle the K range is shared, never below
+// kRows128MinSteps K steps for a workgroup.  Up to 128 rows there is a second way to occupy the idle units: narrower
+// workgroups (5 or 6 waves) with K unshared - a unit's pull covers the X block and the W rows of a step alike, so
+// more, narrower workgroups mean fewer bytes per unit.  It is taken when such a width gives between 0.55 cus and cus
+// tiles (DeepSeek-V3 gate_up, N = 36864: 231 tiles of 160 rows, M = 64 / 128: 50.3 / 62.8 us against 59.4 / 68.8
+// for 144 tiles of 256; q_b, N = 24576, K = 1536: 16.6 against 21.4 with K shared by two).
+struct Rows128Plan {
+    int wv, bn, splits, tiles;
+};
+
+static Rows128Plan rows128_plan(int64_t M, int64_t N, int64_t K, int cus) {
+    Rows128Plan pl;
+    const int64_t KB = K / kBlockK;
+    pl.wv = 8;
+    pl.bn = M <= 128 ? 256 : 128;
+    if (M <= 128) {
+        for (int wv = 5; wv <= 6; ++wv) {
+            const int64_t tiles = (N + 32 * wv - 1) / (32 * wv);
+            if (tiles <= cus && tiles * 20 >= (int64_t)cus * 11) {
+                pl.wv = wv;
+                pl.bn = 32 * wv;
+                pl.splits = 1;
+                pl.tiles = (int)tiles;
+                return pl;
+            }
+        }
+    }
+    const int64_t tiles = (N + pl.bn - 1) / pl.bn;
     int64_t splits = cus / tiles;
     if (splits > KB / kRows128MinSteps) splits = KB / kRows128MinSteps;
-    return (int)(splits < 1 ? 1 : splits);
+    pl.splits = (int)(splits < 1 ? 1 : splits);
+    pl.tiles = (int)tiles;
+    return pl;
 }
 
-static size_t rows128_workspace(int64_t M, int64_t N, int splits) {
-    const int bn = rows128_bn(M);
-    const int64_t tiles = (N + bn - 1) / bn;
-    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 16 * rows128_mt(M) * bn * 4;
+static int rows128_splits(int64_t M, int64_t N, int64_t K, int cus) { return rows128_plan(M, N, K, cus).splits; }
+
+static size_t rows128_workspace(int64_t M, int64_t N, int64_t K, int cus) {
+    const Rows128Plan pl = rows128_plan(M, N, K, cus);
+    if (pl.splits <= 1) return 0;
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)pl.tiles * pl.splits * 16 * rows128_mt(M) * pl.bn * 4;
 }
 
 // Where the kernel pays (Llama-3-8B and DeepSeek-V3 linears, weights rotated so that none is found in the
@@ -365,12 +392,16 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         if (tiles * 2 <= cus) return tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
         return M <= 160 && tiles <= cus;
     }
+    // up to 128 rows: a single well-filled launch always pays (narrow or full-width workgroups on 0.55 cus .. cus
+    // tiles with K unshared: DeepSeek-V3 gate_up at M = 64: 49.7 us against 69.9 - 72.5 for the streaming kernels,
+    // q_b 12.5 against 15.0, Llama-3 gate_up 29.5 against 29.8)
+    const Rows128Plan pl = rows128_plan(M, N, K, cus);
+    if (pl.splits == 1 && pl.tiles <= cus && pl.tiles * 20 >= (int64_t)cus * 11) return true;
     if (M > 64) return K / kBlockK >= 16;
-    if (N * K < 100000000ll) return false;
-    // more tiles than units (lm_head, N = 128256, K = 4096, M = 64: 116 us against 110 for the shared-activation
-    // streaming kernel, whose small workgroups fill the second round better)
-    if ((N + 255) / 256 > cus) return false;
-    return rows128_splits(M, N, K, cus) == 1 || !xshare_pays(M, N, K, cus);
+    // 33..64 rows with K shared or more tiles than units: on the large weights only, and not where the
+    // shared-activation streaming kernel runs (lm_head, N = 128256, K = 4096, M = 64: 116 us against 110 - its small
+    // workgroups fill the second round better)
+    return N * K >= 100000000ll && pl.tiles <= cus && !xshare_pays(M, N, K, cus);
 }
 
 static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t as_m, int64_t as_k, int cus) {
@@ -383,27 +414,38 @@ static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int6
     return Rows128Cfg<8, 3, 2>::lds_bytes((int)steps) <= 160 * 1024;
 }
 
-template <int MT>
-static int launch_rows128(GemmArgs &a, int splits, void *ws, hipStream_t st) {
+template <int MT, int WV>
+static int launch_rows128_as(GemmArgs &a, const Rows128Plan &pl, void *ws, hipStream_t st) {
     constexpr int TN = MT <= 8 ? 2 : 1, NS = MT <= 8 ? 3 : 2;
-    using Cfg = Rows128Cfg<MT, NS, TN>;
+    using Cfg = Rows128Cfg<MT, NS, TN, WV>;
     const int KB = a.K / kBlockK;
-    const int steps = (KB + splits - 1) / splits;
+    const int steps = (KB + pl.splits - 1) / pl.splits;
     const int lds_bytes = Cfg::lds_bytes(steps);
     if (lds_bytes > 160 * 1024) return MI355_EUNSUPPORTED;
-    const int tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
-    if (splits <= 1) {
-        constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, false>;
+    if (pl.splits <= 1) {
+        constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, WV, false>;
         if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
-        return launch(kernel, dim3(tiles), dim3(Cfg::kThreads), lds_bytes, st, a);
+        return launch(kernel, dim3(pl.tiles), dim3(Cfg::kThreads), lds_bytes, st, a);
     }
-    constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, true>;
-    if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
-    a.splits = splits;
-    a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);  // the counter words stay untouched
-    const int r = launch(kernel, dim3(tiles * splits), dim3(Cfg::kThreads), lds_bytes, st, a);
-    if (r != MI355_OK) return r;
-    return launch(rows128_reduce_kernel<MT, TN>, dim3((tiles * Cfg::kWaves * MT + 3) / 4), dim3(256), 0, st, a);
+    if constexpr (WV == 8) {
+        constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, 8, true>;
+        if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
+        a.splits = pl.splits;
+        a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);  // the counter words stay untouched
+        const int r = launch(kernel, dim3(pl.tiles * pl.splits), dim3(Cfg::kThreads), lds_bytes, st, a);
+        if (r != MI355_OK) return r;
+        return launch(rows128_reduce_kernel<MT, TN>, dim3((pl.tiles * Cfg::kWaves * MT + 3) / 4), dim3(256), 0, st, a);
+    }
+    return MI355_EINVAL;  // narrow workgroups never share K
+}
+
+template <int MT>
+static int launch_rows128(GemmArgs &a, const Rows128Plan &pl, void *ws, hipStream_t st) {
+    if constexpr (MT <= 8) {
+        if (pl.wv == 5) return launch_rows128_as<MT, 5>(a, pl, ws, st);
+        if (pl.wv == 6) return launch_rows128_as<MT, 6>(a, pl, ws, st);
+    }
+    return launch_rows128_as<MT, 8>(a, pl, ws, st);
 }
 
 static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n) {
@@ -416,8 +458,9 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 //     of 128 weight rows (cus if M <= 160; above
 //     256 rows only if N*K >= 2e7)                   the weight stream with the activation block in LDS
 //   65 <= M <= 128, K >= 2048                        the same with 256 weight rows per workgroup
-//   33 <= M <= 64, N*K >= 1e8                        the same, unless it would have to share K between workgroups
-//                                                    where the kernel below runs (Llama-3 gate_up: 30.7 us against 29.8)
+//   33 <= M <= 64, N*K >= 1e8, at most cus tiles     the same, unless the kernel below would run
+//   33 <= M <= 128, 0.55 cus .. cus tiles of 160,
+//     192 or 256 weight rows with K unshared          the same, workgroups of that width
 //   M <= 64                                          weight streaming (M > 32 and N/128 about the unit count: the
 //                                                    kernel that shares the activation block in the workgroup)
 //   few 256x256 tiles, long K                        stream-K (the plain loop would leave most units idle)
@@ -478,8 +521,7 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     }
     if (variant == MI355_GEMM_ROWS128) {
         if (M > 384) return 0;
-        const int splits = rows128_splits(M, N, K, cus);
-        return splits > 1 ? rows128_workspace(M, N, splits) : 0;
+        return rows128_workspace(M, N, K, cus);
     }
     if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
     const SkinnyPlan pl = skinny_plan(M, N, K, cus);
@@ -523,7 +565,7 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
         if (variant == MI355_GEMM_ROWS128 &&
             (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus) ||
              (rows128_splits(M, N, K, cus) > 1 &&
-              (!ws || ws_bytes < rows128_workspace(M, N, rows128_splits(M, N, K, cus)) || ((uintptr_t)ws & 15)))))
+              (!ws || ws_bytes < rows128_workspace(M, N, K, cus) || ((uintptr_t)ws & 15)))))
             variant = pick_variant(M, N, K, cus, false);
         if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
             variant = MI355_GEMM_TILE128;
@@ -602,34 +644,34 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
         }
         case MI355_GEMM_ROWS128: {
             if (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus)) return MI355_EUNSUPPORTED;
-            const int splits = rows128_splits(M, N, K, cus);
-            if (splits > 1 && (!ws || ws_bytes < rows128_workspace(M, N, splits) || ((uintptr_t)ws & 15)))
+            const Rows128Plan pl = rows128_plan(M, N, K, cus);
+            if (pl.splits > 1 && (!ws || ws_bytes < rows128_workspace(M, N, K, cus) || ((uintptr_t)ws & 15)))
                 return MI355_EWORKSPACE;
             switch (rows128_mt(M)) {
-                case 1: return launch_rows128<1>(a, splits, ws, st);
-                case 2: return launch_rows128<2>(a, splits, ws, st);
-                case 3: return launch_rows128<3>(a, splits, ws, st);
-                case 4: return launch_rows128<4>(a, splits, ws, st);
-                case 5: return launch_rows128<5>(a, splits, ws, st);
-                case 6: return launch_rows128<6>(a, splits, ws, st);
-                case 7: return launch_rows128<7>(a, splits, ws, st);
-                case 8: return launch_rows128<8>(a, splits, ws, st);
-                case 9: return launch_rows128<9>(a, splits, ws, st);
-                case 10: return launch_rows128<10>(a, splits, ws, st);
-                case 11: return launch_rows128<11>(a, splits, ws, st);
-                case 12: return launch_rows128<12>(a, splits, ws, st);
-                case 13: return launch_rows128<13>(a, splits, ws, st);
-                case 14: return launch_rows128<14>(a, splits, ws, st);
-                case 15: return launch_rows128<15>(a, splits, ws, st);
-                case 16: return launch_rows128<16>(a, splits, ws, st);
-                case 17: return launch_rows128<17>(a, splits, ws, st);
-                case 18: return launch_rows128<18>(a, splits, ws, st);
-                case 19: return launch_rows128<19>(a, splits, ws, st);
-                case 20: return launch_rows128<20>(a, splits, ws, st);
-                case 21: return launch_rows128<21>(a, splits, ws, st);
-                case 22: return launch_rows128<22>(a, splits, ws, st);
-                case 23: return launch_rows128<23>(a, splits, ws, st);
-                default: return launch_rows128<24>(a, splits, ws, st);
+                case 1: return launch_rows128<1>(a, pl, ws, st);
+                case 2: return launch_rows128<2>(a, pl, ws, st);
+                case 3: return launch_rows128<3>(a, pl, ws, st);
+                case 4: return launch_rows128<4>(a, pl, ws, st);
+                case 5: return launch_rows128<5>(a, pl, ws, st);
+                case 6: return launch_rows128<6>(a, pl, ws, st);
+                case 7: return launch_rows128<7>(a, pl, ws, st);
+                case 8: return launch_rows128<8>(a, pl, ws, st);
+                case 9: return launch_rows128<9>(a, pl, ws, st);
+                case 10: return launch_rows128<10>(a, pl, ws, st);
+                case 11: return launch_rows128<11>(a, pl, ws, st);
+                case 12: return launch_rows128<12>(a, pl, ws, st);
+                case 13: return launch_rows128<13>(a, pl, ws, st);
+                case 14: return launch_rows128<14>(a, pl, ws, st);
+                case 15: return launch_rows128<15>(a, pl, ws, st);
+                case 16: return launch_rows128<16>(a, pl, ws, st);
+                case 17: return launch_rows128<17>(a, pl, ws, st);
+                case 18: return launch_rows128<18>(a, pl, ws, st);
+                case 19: return launch_rows128<19>(a, pl, ws, st);
+                case 20: return launch_rows128<20>(a, pl, ws, st);
+                case 21: return launch_rows128<21>(a, pl, ws, st);
+                case 22: return launch_rows128<22>(a, pl, ws, st);
+                case 23: return launch_rows128<23>(a, pl, ws, st);
+                default: return launch_rows128<24>(a, pl, ws, st);
             }
         }
         case MI355_GEMM_SKINNY: {

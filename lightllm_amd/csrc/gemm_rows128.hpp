@@ -7,8 +7,8 @@
 //
 //   16*MT activation rows (MT MFMA row blocks) x 128*TN weight rows, K step 128.
 //     TN = 2: up to 128 rows (MT <= 8) against 256 weight rows; TN = 1: up to 384 rows (MT <= 24) against 128.
-//   8 waves, wave w owns 16*TN weight rows and all activation rows: MT x TN MFMA blocks per K step (the X operand
-//   blocks are read from LDS eight at a time).
+//   WV waves (8; fewer for some unsplit launches, see below), wave w owns 16*TN weight rows and all activation rows:
+//   MT x TN MFMA blocks per K step (the X operand blocks are read from LDS eight at a time).
 //   NS ring slots of { X 16*MT x 128 B, W 128*TN x 128 B }.  A wave fetches its own W rows (2*TN requests of 1 KiB
 //   per step) into its own part of a slot and is the only one to read them, so the W stream needs no barrier: the rows
 //   of step kb + NS are requested as soon as the wave has read those of step kb.  The X block is shared: one barrier
@@ -20,6 +20,10 @@
 //   16*MT x 128*TN floats each, too many for the last workgroup of a tile to add alone (one compute unit reads
 //   about 40 GB/s): they go to the workspace and a second, device-wide launch adds them in split order.
 //
+//   What a unit pulls is X and W together - the X block comes from L2, but through the same requests - so a launch
+//   whose 256-row tiles leave units idle and whose K cannot be shared usefully runs narrower workgroups instead
+//   (WV = 5 or 6: 160 or 192 weight rows), as many as there are units: every unit then loads less per K step.
+//
 //   (Half-width tiles of four waves on two slots, two workgroups to a unit, were tried for shapes whose 256-row
 //   tiles leave units idle and cannot share K usefully - N = 36864: 144 tiles on 256 units - and were slower: 85 us
 //   against 69 at M = 128.)
@@ -30,11 +34,11 @@
 
 namespace mi355 {
 
-template <int MT, int NS, int TN_ = 2>
+template <int MT, int NS, int TN_ = 2, int WV = 8>
 struct Rows128Cfg {
-    static_assert(MT >= 1 && MT <= (TN_ == 2 ? 8 : 24) && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
-    static constexpr int TN = TN_, WNS = 16 * TN, kWaves = 8, kThreads = 512, BN = WNS * kWaves;
-    static constexpr int NBLK = (BN + kBlockN - 1) / kBlockN;  // 128-wide n blocks of a tile
+    static_assert(WV >= 4 && WV <= 8 && MT >= 1 && MT <= (TN_ == 2 ? 8 : 24) && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
+    static constexpr int TN = TN_, WNS = 16 * TN, kWaves = WV, kThreads = 64 * WV, BN = WNS * WV;
+    static constexpr int NBLK = (BN + 2 * kBlockN - 2) / kBlockN;  // 128-wide n blocks a tile can touch
     static constexpr int NWW = 2 * TN;                         // W requests per wave and step (8 rows each)
     static constexpr int XG = 2 * MT;                          // 8-row request groups of the X block
     static constexpr int NXW = (XG + kWaves - 1) / kWaves;     // X requests per wave (groups repeat if XG % 8 != 0)
@@ -66,9 +70,9 @@ __device__ __forceinline__ void rows128_store(const GemmArgs &p, int row, int nb
     }
 }
 
-template <int MT, int NS, int TN, bool SPLIT>
-__global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmArgs p) {
-    using Cfg = Rows128Cfg<MT, NS, TN>;
+template <int MT, int NS, int TN, int WV, bool SPLIT>
+__global__ __launch_bounds__(64 * WV) void block_fp8_gemm_rows128_kernel(const GemmArgs p) {
+    using Cfg = Rows128Cfg<MT, NS, TN, WV>;
     constexpr int WNS = Cfg::WNS, NXW = Cfg::NXW, XG = Cfg::XG, NWW = Cfg::NWW, XH = Cfg::XH;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -162,11 +166,11 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
         const int NBk = (p.N + kBlockN - 1) / kBlockN;
         float *wl = (float *)(lds + Cfg::kWsOff);
         for (int i = tid; i < Cfg::NBLK * steps; i += Cfg::kThreads) {
-            const int b = i >= steps ? 1 : 0, it = i - b * steps;
+            const int b = i / steps, it = i - b * steps;
             wl[i] = p.Ws[(int64_t)min(n0 / kBlockN + b, NBk - 1) * p.ws_n + (int64_t)(kb_begin + it) * p.ws_k];
         }
     }
-    const float *wsl = (const float *)(lds + Cfg::kWsOff) + ((wave * WNS) / kBlockN) * steps;
+    const float *wsl = (const float *)(lds + Cfg::kWsOff) + ((n0 + wave * WNS) / kBlockN - n0 / kBlockN) * steps;
 
     v4f acc[MT][TN];
 #pragma unroll
@@ -265,7 +269,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_rows128_kernel(const GemmA
 // splits in split order and stores 4*TN consecutive outputs of row 16*i + lane % 16.
 template <int MT, int TN>
 __global__ __launch_bounds__(256) void rows128_reduce_kernel(const GemmArgs p) {
-    using Cfg = Rows128Cfg<MT, 2, TN>;
+    using Cfg = Rows128Cfg<MT, 2, TN, 8>;  // K is shared between 8-wave workgroups only
     constexpr int WNS = Cfg::WNS, F = MT * TN;
     const int lane = threadIdx.x & 63;
     const int item = blockIdx.x * 4 + (threadIdx.x >> 6);  // (tile, wave, i)

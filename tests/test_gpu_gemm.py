@@ -243,7 +243,8 @@ def test_shared_activation_stream_kernel(hip):
                                               ws.cpu().numpy(), np.arange(len(rows)), cols)
         got = c[rows][:, cols].float().cpu().double().numpy()
         assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
-    xq, xs, wq, ws = _prep(64, 28672, 4096, seed=77, device="cuda")
+    # the table sends 33..64 rows there when N alone gives more 256-row tiles than compute units
+    xq, xs, wq, ws = _prep(64, 66048, 1024, seed=77, device="cuda")
     assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), _run(xq, xs, wq, ws, "xshare").view(torch.int16))
 
 
@@ -262,6 +263,7 @@ def test_rows128_stream_kernel(hip):
     cases += [(int(rng.integers(129, 385)), int(rng.integers(1, 300)) * int(rng.choice([1, 4, 8, 16, 128])),
                int(rng.choice([128, 256, 640, 1024, 2048, 7168, 18432]))) for _ in range(18)]
     cases += [(128, 256, 128), (65, 4096, 14336), (127, 2112, 7168), (80, 520, 2304), (256, 128, 128), (129, 7168, 2048),
+              (100, 160 * 200 + 8, 640), (40, 192 * 230 - 3, 512), (128, 160 * 141, 256),   # 160- and 192-row workgroups
               (255, 2112, 7168), (144, 1000, 4096), (384, 640, 4096), (257, 136, 256), (383, 4100, 2048)]
     shared = 0
     for case, (M, N, K) in enumerate(cases):
@@ -301,7 +303,8 @@ def test_rows128_column_major_scales(hip):
 
 @pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
                                    (128, 2112, 7168), (256, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
-                                   (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384)])
+                                   (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384), (48, 24576, 1536),
+                                   (64, 28672, 4096)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
     """Model linears with 33..384 rows that the shape table gives to the weight stream with the activation block in
     LDS."""
