@@ -453,6 +453,21 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
            ((uintptr_t)B & 15) == 0;
 }
 
+// 256x128 tiles that are too few to occupy the device share the K range the same way.
+static int tile256x128_splits(int64_t M, int64_t N, int64_t K, int cus) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
+    const int64_t KB = K / kBlockK;
+    if (tiles * 2 > cus || KB < 16) return 1;
+    int64_t splits = cus / tiles;
+    if (splits > KB / 8) splits = KB / 8;
+    return (int)(splits < 1 ? 1 : splits);
+}
+
+static size_t tile256x128_workspace(int64_t M, int64_t N, int splits) {
+    const int64_t tiles = ((M + 255) / 256) * ((N + 127) / 128);
+    return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 256 * 128 * 4;
+}
+
 // The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
 //   129 <= M <= 384, K >= 2048, at most cus/2 tiles
 //     of 128 weight rows (cus if M <= 160; above
@@ -466,6 +481,7 @@ static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda,
 //   few 256x256 tiles, long K                        stream-K (the plain loop would leave most units idle)
 //   128x128 tiles fit one round of two per unit and
 //     (few 256x256 tiles or a short K)               128x128 tiles, K shared between workgroups when they are few
+//                                                    (M >= 768 and N <= 3072: 256x128 tiles with K shared)
 //   otherwise                                        256x256 ping-pong tiles
 static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_rows128 = true) {
     if (allow_rows128 && rows128_pays(M, N, K, cus)) return MI355_GEMM_ROWS128;
@@ -475,7 +491,13 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
     const int64_t KB = K / kBlockK;
     if (M > 128 && stream_k_pays(t256, KB, cus)) return MI355_GEMM_TILE256_STREAMK;
-    if (t128 <= 2 * (int64_t)cus && (t256 < (int64_t)cus * 3 / 8 || KB <= 64)) return MI355_GEMM_TILE128;
+    if (t128 <= 2 * (int64_t)cus && (t256 < (int64_t)cus * 3 / 8 || KB <= 64)) {
+        // a narrow N under many rows: 256x128 tiles with K shared load half as much X per product as the 128x128
+        // ones and still fill the device (q_a+kv_a, N = 2112, K = 7168, M = 768 / 1024 / 1536: 35.0 / 40.6 / 50.6 us
+        // against 38.7 / 60.2 / 60.6)
+        if (M >= 768 && (N + 127) / 128 <= 24 && tile256x128_splits(M, N, K, cus) >= 2) return MI355_GEMM_TILE256x128;
+        return MI355_GEMM_TILE128;
+    }
     if (t256 >= (int64_t)cus * 3 / 8) return MI355_GEMM_TILE256;
     return MI355_GEMM_TILE128;
 }
@@ -513,6 +535,10 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     if (variant == MI355_GEMM_TILE128) {
         const int splits = tile128_splits(M, N, K, cus);
         return splits > 1 ? tile128_workspace(M, N, splits) : 0;
+    }
+    if (variant == MI355_GEMM_TILE256x128) {
+        const int splits = tile256x128_splits(M, N, K, cus);
+        return splits > 1 ? tile256x128_workspace(M, N, splits) : 0;
     }
     if (variant == MI355_GEMM_TILE256) return MI355_WS_COUNTER_BYTES;  // the tile counters of the persistent launch
     if (variant == MI355_GEMM_SKINNY_XSHARE) {
@@ -617,8 +643,18 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
         }
         case MI355_GEMM_TILE256_RING:  // kept for comparison
             return launch_dense<256, 256, 2, 4, 2>(a, st);
-        case MI355_GEMM_TILE256x128:
-            return launch_dense<256, 128, 2, 4, 3>(a, st);
+        case MI355_GEMM_TILE256x128: {
+            const int splits = tile256x128_splits(M, N, K, cus);
+            if (splits <= 1 || !ws || ws_bytes < tile256x128_workspace(M, N, splits) || ((uintptr_t)ws & 15))
+                return launch_dense<256, 128, 2, 4, 3>(a, st);
+            a.tiles_m = (a.M + 255) / 256;
+            a.tiles_n = (a.N + 127) / 128;
+            a.total_tiles = a.tiles_m * a.tiles_n;
+            a.splits = splits;
+            a.counters = (uint32_t *)ws;
+            a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+            return launch_tile<256, 128, 2, 4, 3, kSplitK>(a, a.total_tiles * splits, st);
+        }
         case MI355_GEMM_TILE128: {
             const int splits = tile128_splits(M, N, K, cus);
             if (splits <= 1 || !ws || ws_bytes < tile128_workspace(M, N, splits) || ((uintptr_t)ws & 15))

@@ -373,6 +373,30 @@ def test_mid_m_split_k_tiles(hip, M, N, K):
     assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("M,N,K", [(768, 2112, 7168), (1024, 2112, 7168), (300, 520, 4096)])
+def test_256x128_tiles_with_shared_k(hip, M, N, K):
+    """256x128 tiles whose K range is shared between workgroups (few tiles, long K): against the torch fp32
+    dequant-matmul, the float64 oracle on a sample and the 128x128 tiles; repeated calls agree bit for bit.  The
+    shape table sends narrow-N shapes with many rows there."""
+    from lightllm_amd import _lib
+
+    print(f"gemm 256x128 split-K M={M} N={N} K={K}", flush=True)
+    assert _lib.lib().mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_TILE256x128) > 0
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + K)
+    C1 = _run(xq, xs, wq, ws, "tile256x128").clone()
+    assert torch.equal(C1, _run(xq, xs, wq, ws, "tile256x128"))
+    if M >= 768:
+        assert torch.equal(C1, _run(xq, xs, wq, ws, None))
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(C1.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+    assert (C1.float() - _run(xq, xs, wq, ws, "tile128").float()).abs().max() <= ref.abs().max() * 2 ** -7
+    rows, cols = np.arange(0, M, 37), np.arange(0, N, 11)
+    ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq), xs.cpu().numpy(), tr.bits_of(wq), ws.cpu().numpy(), rows, cols)
+    got = C1[rows][:, cols].float().cpu().double().numpy()
+    assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
+
+
 def test_split_k_is_deterministic_and_reusable(hip):
     """The split-K path reduces in a fixed order and leaves its workspace counters zero: repeated calls agree bit for bit."""
     print("gemm split-k determinism", flush=True)
