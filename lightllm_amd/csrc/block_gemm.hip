@@ -491,6 +491,9 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
     const int64_t KB = K / kBlockK;
     if (M > 128 && stream_k_pays(t256, KB, cus)) return MI355_GEMM_TILE256_STREAMK;
+    // 257..384 rows leave the second 256-row tile at most half full; where the 256x256 tiles need a second round
+    // anyway the 128x128 ones are ahead (N = 36864, K = 7168, M = 257 / 384: 144 / 148 us against 161 / 165)
+    if (M > 256 && M <= 384 && t256 > cus && t128 <= 4 * (int64_t)cus) return MI355_GEMM_TILE128;
     if (t128 <= 2 * (int64_t)cus && (t256 < (int64_t)cus * 3 / 8 || KB <= 64)) {
         // a narrow N under many rows: 256x128 tiles with K shared load half as much X per product as the 128x128
         // ones and still fill the device (q_a+kv_a, N = 2112, K = 7168, M = 768 / 1024 / 1536: 35.0 / 40.6 / 50.6 us
