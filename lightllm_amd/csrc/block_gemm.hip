@@ -76,7 +76,7 @@ static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
 // the tiles fill whole rounds anyway or there is too little work to give every unit 16 K steps (the 128x128
 // split-K tiles take those shapes).
 static int stream_k_groups(int64_t tiles, int64_t KB, int cus) {
-    if (cus < 8 || tiles <= 0 || tiles > 16384 - PPCfg::kTileCounterWord) return 0;
+    if (cus < 8 || tiles <= 0) return 0;
     const int64_t units = tiles * KB;
     if (units >= (1ll << 31)) return 0;
     const int64_t groups = cus / 8 * 8;
@@ -125,8 +125,11 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, int sk_gro
             if (!ws_ok || ws_bytes < stream_k_workspace(sk_groups)) return MI355_EWORKSPACE;
             a.counters = (uint32_t *)ws;
             a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
-            return sc4 ? launch_pp_as<false, true, true>(a, sk_groups, lds_bytes, st)
-                       : launch_pp_as<false, true, false>(a, sk_groups, lds_bytes, st);
+            const int r = sc4 ? launch_pp_as<false, true, true>(a, sk_groups, lds_bytes, st)
+                              : launch_pp_as<false, true, false>(a, sk_groups, lds_bytes, st);
+            if (r != MI355_OK) return r;
+            return launch(streamk_reduce_kernel, dim3(a.total_tiles * PPCfg::TM), dim3(PPCfg::kThreads), 0, st, a,
+                          (uint32_t)sk_groups);
         }
     }
     // persistent only when there is more than one tile per CU (a single round gains nothing from the tile queue)

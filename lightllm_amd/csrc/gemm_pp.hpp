@@ -33,9 +33,9 @@
 //     tiles - tile-major, in the dense tile order - are cut into one contiguous run per workgroup, so every compute
 //     unit does the same number of K steps.  A workgroup whose run covers only part of a tile's K range writes its
 //     fp32 accumulators to its own slot of the workspace (two slots per workgroup: a run starts and ends inside at
-//     most one tile each) and bumps the tile's arrival counter; whoever arrives last adds the tile's partials in K
-//     order (so the result does not depend on who that is), stores the tile and re-zeroes the counter.  Nobody
-//     waits for anybody.
+//     most one tile each); a second launch (streamk_reduce_kernel) adds the parts of every shared tile in K order
+//     and stores it.  (Adding them in the last workgroup to arrive at a tile was 3 to 8 % slower: one compute unit
+//     reads the parts of a tile at a fraction of the rate the whole device does.)
 //   * ROLES (grouped launch with a workspace): schedule blocks with at most 64 rows are weight streams, and this
 //     tile streams badly (32 KiB of W in flight per step, three quarters of the X area and half of the waves
 //     idle).  They go to the 64 x 512 tile of gemm_small.hpp instead, in the same launch: a split kernel has
@@ -71,7 +71,6 @@ struct PPCfg {
     static constexpr int roles_sched_off(int KB) {
         return sched_off(KB) > SmallCfg::lds_bytes(KB) ? sched_off(KB) : SmallCfg::lds_bytes(KB);
     }
-    static constexpr int kTileCounterWord = 16;       // stream-K: arrival counters of the tiles start here
     static constexpr int kPartialBytes = BM * BN * 4;  // one fp32 partial tile
 };
 
@@ -496,7 +495,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
             ws_first = ws_load(cur);
         }
 
-        // ---- stream-K: a part of a tile goes to the workspace; the last part to arrive adds them all up
+        // ---- stream-K: a part of a tile goes to the workspace
         bool store_tile = true;
         if constexpr (SK) {
             if (done.k0 != 0 || done.k1 != KB) {  // the same for the whole workgroup
@@ -508,43 +507,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) xch.store(mine + (uint32_t)(i * TN + j) * kBlockStride, acc[i][j]);
-                wait_vmcnt<0>();
-                __syncthreads();
-                // the ranks that hold parts of this tile: those whose runs contain its first and its last unit
-                const uint64_t t0 = (uint64_t)done.id * (uint64_t)KB;
-                const uint32_t r_lo = (uint32_t)(((t0 + 1u) * gridDim.x - 1u) / units);
-                const uint32_t r_hi = (uint32_t)(((t0 + (uint64_t)KB) * gridDim.x - 1u) / units);
-                uint32_t *counter = p.counters + Cfg::kTileCounterWord + done.id;
-                if (tid == 0) sched[0] = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __syncthreads();
-                store_tile = sched[0] == r_hi - r_lo;
-                if (store_tile) {
-                    // parts in K order: the first rank's run ends inside the tile (its second slot), every later
-                    // one starts inside it (its first slot).  The first part is loaded straight into the
-                    // accumulators, the others in halves.
-                    const uint32_t first = (2u * r_lo + 1u) * (uint32_t)Cfg::kPartialBytes + lane_off;
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-#pragma unroll
-                        for (int j = 0; j < TN; ++j) acc[i][j] = xch.load(first + (uint32_t)(i * TN + j) * kBlockStride);
-                    for (uint32_t r = r_lo + 1; r <= r_hi; ++r) {
-                        const uint32_t src = 2u * r * (uint32_t)Cfg::kPartialBytes + lane_off;
-#pragma unroll
-                        for (int h = 0; h < 2; ++h) {
-                            v4f part[TM / 2][TN];
-#pragma unroll
-                            for (int i = 0; i < TM / 2; ++i)
-#pragma unroll
-                                for (int j = 0; j < TN; ++j)
-                                    part[i][j] = xch.load(src + (uint32_t)((h * (TM / 2) + i) * TN + j) * kBlockStride);
-#pragma unroll
-                            for (int i = 0; i < TM / 2; ++i)
-#pragma unroll
-                                for (int j = 0; j < TN; ++j) acc[h * (TM / 2) + i][j] += part[i][j];
-                        }
-                    }
-                    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+                store_tile = false;  // the second launch (streamk_reduce_kernel) adds the parts and stores the tile
             }
         }
 
@@ -607,6 +570,64 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
 #pragma unroll
             for (int i = 0; i < Cfg::kCounterWords; ++i)
                 __hip_atomic_store(p.counters + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+// Second launch of a stream-K GEMM: workgroup (tile, row block i) adds the parts of the tile that
+// the first launch left in the workspace - in K order, so the result does not depend on the schedule - and stores
+// the 16-row slices 16*i + [0, 16) of both wave rows.  Tiles that one workgroup computed whole were stored by it.
+// `groups` is the grid size of the first launch.
+__global__ __launch_bounds__(512) void streamk_reduce_kernel(const GemmArgs p, uint32_t groups) {
+    using Cfg = PPCfg;
+    constexpr int TN = Cfg::TN, WMS = Cfg::WMS, WNS = Cfg::WNS;
+    constexpr uint32_t kBlockStride = Cfg::kThreads * 16;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave >> 2, wave_n = wave & 3, r16 = lane & 15, g4 = lane >> 4;
+    const uint32_t id = blockIdx.x / Cfg::TM, i = blockIdx.x % Cfg::TM;
+    const uint32_t KB = (uint32_t)(p.K / kBlockK);
+    const uint64_t units = (uint64_t)p.total_tiles * KB, t0 = (uint64_t)id * KB;
+    const uint32_t r_lo = (uint32_t)(((t0 + 1u) * groups - 1u) / units);
+    const uint32_t r_hi = (uint32_t)(((t0 + (uint64_t)KB) * groups - 1u) / units);
+    if (r_lo == r_hi) return;
+    // parts in K order: the first rank's run ends inside the tile (its second slot), every later one starts
+    // inside it (its first slot)
+    const uint8_t *base = (const uint8_t *)p.partials + (uint32_t)tid * 16u + i * TN * kBlockStride;
+    v4f acc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+        acc[j] = *(const v4f *)(base + (uint64_t)(2u * r_lo + 1u) * Cfg::kPartialBytes + (uint32_t)j * kBlockStride);
+    for (uint32_t r = r_lo + 1; r <= r_hi; ++r) {
+        v4f part[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) part[j] = *(const v4f *)(base + (uint64_t)(2u * r) * Cfg::kPartialBytes + (uint32_t)j * kBlockStride);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[j] += part[j];
+    }
+    constexpr uint32_t GM = 8;
+    const uint32_t width = GM * (uint32_t)p.tiles_n, g = id / width, first_m = g * GM;
+    const uint32_t gsz = min((uint32_t)p.tiles_m - first_m, GM), in_grp = id - g * width;
+    const int m0 = (int)(first_m + in_grp % gsz) * Cfg::BM, n0 = (int)(in_grp / gsz) * Cfg::BN;
+    const int rl = wave_m * WMS + 16 * (int)i + r16;
+    if (m0 + rl >= p.M) return;
+    const int nbase = n0 + wave_n * WNS;
+    uint16_t *cp = p.C + (int64_t)(m0 + rl) * p.ldc + nbase;
+    float o[4 * TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = acc[j][vv];
+    if (p.vec_store && nbase + WNS <= p.N) {
+#pragma unroll
+        for (int h = 0; h < TN / 2; ++h)
+            *(v4i *)(cp + lane_col<TN>(g4, 2 * h)) =
+                v4i{(int)pack_out2(o[8 * h + 0], o[8 * h + 1], p.out_f16), (int)pack_out2(o[8 * h + 2], o[8 * h + 3], p.out_f16),
+                    (int)pack_out2(o[8 * h + 4], o[8 * h + 5], p.out_f16), (int)pack_out2(o[8 * h + 6], o[8 * h + 7], p.out_f16)};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4 * TN; ++e) {
+            const int c = lane_col<TN>(g4, e >> 2) + (e & 3);
+            if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
         }
     }
 }
