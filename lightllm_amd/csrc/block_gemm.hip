@@ -524,6 +524,20 @@ static size_t tile128_workspace(int64_t M, int64_t N, int splits) {
     return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 128 * 128 * 4;
 }
 
+// A launch of 256x256 tiles that fills the device once and leaves a small rest for a second round runs the rest
+// as a launch of its own, with whatever the table gives its shape (mostly 128x128 tiles, which spread it over the
+// whole device): N = 36864, K = 7168, M = 512 (288 tiles on 256 units) 137 us against 169; q_b, M = 768, 43.6
+// against 50.2.  With two or more full rounds, or a rest of more than half a round, it gains nothing.  Returns the
+// number of weight rows of the first launch, 0 for no split.
+static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus) {
+    (void)K;
+    const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256, t256 = tiles_m * tiles_n;
+    if (tiles_m > cus || t256 <= cus || t256 >= 2 * (int64_t)cus) return 0;
+    if ((t256 - cus) * 2 > cus) return 0;
+    const int64_t n1 = (int64_t)cus / tiles_m * 256;
+    return n1 > 0 && n1 < N ? n1 : 0;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -533,7 +547,14 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     if (K % kBlockK != 0) return 0;
     // sized from the launch plan of the current device (256 compute units when no device is visible)
     const int cus = device_cus();
-    if (variant == MI355_GEMM_AUTO) variant = pick_variant(M, N, K, cus);
+    if (variant == MI355_GEMM_AUTO) {
+        variant = pick_variant(M, N, K, cus);
+        const int64_t n1 = variant == MI355_GEMM_TILE256 ? n_split_rows(M, N, K, cus) : 0;
+        if (n1 > 0) {
+            const size_t rest = mi355_block_fp8_gemm_workspace_bytes(M, N - n1, K, MI355_GEMM_AUTO);
+            return rest > (size_t)MI355_WS_COUNTER_BYTES ? rest : (size_t)MI355_WS_COUNTER_BYTES;
+        }
+    }
     if (variant == MI355_GEMM_TILE256_STREAMK) {
         const int groups = stream_k_groups(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus);
         return groups > 0 ? stream_k_workspace(groups) : (size_t)MI355_WS_COUNTER_BYTES;
@@ -601,6 +622,17 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
             variant = pick_variant(M, N, K, cus, false);
         if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
             variant = MI355_GEMM_TILE128;
+    }
+    if (was_auto && variant == MI355_GEMM_TILE256) {
+        const int64_t n1 = n_split_rows(M, N, K, cus);
+        if (n1 > 0 && ldb_n * n1 % 16 == 0) {
+            const int r = block_fp8_gemm_impl(A, B, As, Bs, C, M, n1, K, lda, ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n,
+                                              block_n, block_k, ws, ws_bytes, MI355_GEMM_TILE256, c_dtype, stream);
+            if (r != MI355_OK) return r;
+            return block_fp8_gemm_impl(A, (const uint8_t *)B + n1 * ldb_n, As, Bs + n1 / kBlockN * bs_n,
+                                       (uint16_t *)C + n1, M, N - n1, K, lda, ldb_k, ldb_n, ldc, as_m, as_k, bs_k, bs_n,
+                                       block_n, block_k, ws, ws_bytes, MI355_GEMM_AUTO, c_dtype, stream);
+        }
     }
     if (variant != MI355_GEMM_GENERIC && !fast) return MI355_EALIGN;
 

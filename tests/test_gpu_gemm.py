@@ -397,6 +397,40 @@ def test_256x128_tiles_with_shared_k(hip, M, N, K):
     assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
 
 
+@pytest.mark.parametrize("M,N,K", [(512, 36864, 1024), (400, 36864 + 72, 2048), (768, 24576, 1536)])
+def test_rest_of_a_round_runs_as_its_own_launch(hip, M, N, K):
+    """256x256 tiles that fill the device once and leave a small rest: the table runs the rest (the last weight
+    rows) as a second launch with the kernel its own shape gets.  Same products in the same order per output as
+    the one-launch 256x256 tiles when that kernel does not share K, close to it otherwise; fp32 reference and
+    float64 oracle as everywhere."""
+    from lightllm_amd import _lib
+
+    print(f"gemm rest-of-a-round split M={M} N={N} K={K}", flush=True)
+    cus = _lib.device_info()["compute_units"]
+    t256 = -(-M // 256) * -(-N // 256)
+    if not (cus < t256 <= cus * 3 // 2):
+        pytest.skip("shape chosen for 256 compute units")
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + K)
+    c = _run(xq, xs, wq, ws, None).clone()
+    assert not torch.isnan(c.float()).any()
+    assert torch.equal(c, _run(xq, xs, wq, ws, None))
+    one = _run(xq, xs, wq, ws, "tile256")
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    if K // 128 < 16:
+        assert torch.equal(c.view(torch.int16), one.view(torch.int16))
+    else:
+        assert (c.float() - one.float()).abs().max() <= ref.abs().max() * 2 ** -7
+    cos, rel = H.gemm_metrics(c.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+    rng = np.random.default_rng(M)
+    rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 6)])
+    cols = np.unique(np.r_[0, N - 1, N - 4096, N - 4097, rng.integers(0, N, 60)])
+    ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                          ws.cpu().numpy(), np.arange(len(rows)), cols)
+    got = c[rows][:, cols].float().cpu().double().numpy()
+    assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * np.abs(ref64).max()
+
+
 def test_split_k_is_deterministic_and_reusable(hip):
     """The split-K path reduces in a fixed order and leaves its workspace counters zero: repeated calls agree bit for bit."""
     print("gemm split-k determinism", flush=True)
