@@ -509,6 +509,42 @@ def test_generic_strides(hip):
     _check_small(xq, xs, wq, ws, C2)
 
 
+@pytest.mark.parametrize("variant,M,N,K", [("rows128", 100, 1000, 2048), ("rows128", 300, 640, 4096), ("rows128", 64, 160 * 150, 256),
+                                           ("tile128", 200, 520, 4096), ("tile256", 300, 520, 1024), ("tile256x128", 768, 520, 4096),
+                                           ("skinny", 20, 1000, 4096), ("xshare", 40, 4096, 1024), ("tile256streamk", 600, 1024, 8192),
+                                           (None, 512, 36864, 256)])
+def test_padded_rows_through_the_c_abi(hip, variant, M, N, K):
+    """Operands whose rows are longer than they need be (lda > K, ldb_n > K, ldc > N, padded scale rows), as a
+    caller that slices larger buffers passes them: every fast kernel against its own result on packed operands
+    (same kernel, same order: bit-equal), and nothing written into the padding of C."""
+    from lightllm_amd import _lib
+    from lightllm_amd.quantization.fp8w8a8_block_gemm_kernel import _VARIANTS
+
+    print(f"gemm padded rows variant={variant} M={M} N={N} K={K}", flush=True)
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + N)
+    want = _run(xq, xs, wq, ws, variant).clone()
+    xq_p = torch.zeros((M, K + 128), dtype=torch.uint8, device="cuda")
+    xq_p[:, :K] = xq.view(torch.uint8)
+    wq_p = torch.zeros((N, K + 256), dtype=torch.uint8, device="cuda")
+    wq_p[:, :K] = wq.view(torch.uint8)
+    xs_p = torch.zeros((M, K // 128 + 3), dtype=torch.float32, device="cuda")
+    xs_p[:, :K // 128] = xs
+    ws_p = torch.zeros((ws.shape[0], K // 128 + 5), dtype=torch.float32, device="cuda")
+    ws_p[:, :K // 128] = ws
+    out = torch.full((M, N + 8), 7.0, dtype=torch.bfloat16, device="cuda")
+    code = _VARIANTS[variant]
+    need = hip.mi355_block_fp8_gemm_workspace_bytes(M, N, K, code)
+    wsp = torch.zeros(max(need, 16), dtype=torch.uint8, device="cuda")
+    rc = hip.mi355_block_fp8_gemm(xq_p.data_ptr(), wq_p.data_ptr(), xs_p.data_ptr(), ws_p.data_ptr(), out.data_ptr(), M, N, K,
+                                  xq_p.stride(0), 1, wq_p.stride(0), out.stride(0), xs_p.stride(0), 1, 1, ws_p.stride(0),
+                                  128, 128, wsp.data_ptr(), wsp.numel(), code, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0, hip.mi355_error_string(rc)
+    assert torch.equal(out[:, :N].contiguous().view(torch.int16), want.view(torch.int16))
+    assert bool((out[:, N:] == 7.0).all())
+    assert not bool(wsp[:_lib.WS_COUNTER_BYTES].any()) if need >= _lib.WS_COUNTER_BYTES else True
+
+
 def test_preconditions(hip):
     from lightllm_amd.quantization import w8a8_block_fp8_matmul
 
