@@ -92,7 +92,8 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
  * As  fp32 [M, K/block_k]   element (m,kb) at As[m*as_m + kb*as_k]
  * Bs  fp32 [K/block_k, ceil(N/block_n)] element (kb,nb) at Bs[kb*bs_k + nb*bs_n]   (w8a8.py:443: strides (1, K/128))
  * C   bf16 [M,N], row stride ldc, unit column stride (:152)
- * block_n = block_k = 128.
+ * block_n = block_k = 128 for the tiled kernels; any other positive block sizes run on the plain kernel
+ * (MI355_GEMM_AUTO or MI355_GEMM_GENERIC), the last K block may be partial.
  *
  * `variant` picks the kernel: MI355_GEMM_AUTO applies the built-in shape table (and falls back to
  * MI355_GEMM_TILE128 when a limit of the streaming kernel - 32-bit row offsets, workspace - is not met); the

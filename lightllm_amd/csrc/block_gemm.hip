@@ -589,7 +589,10 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
     if (M < 0 || N < 0 || K < 0) return MI355_EINVAL;
     if (c_dtype != MI355_DTYPE_BF16 && c_dtype != MI355_DTYPE_F16) return MI355_EUNSUPPORTED;
     const int out_f16 = c_dtype == MI355_DTYPE_F16 ? 1 : 0;
-    if (block_n != kBlockN || block_k != kBlockK) return MI355_EUNSUPPORTED;
+    if (block_n <= 0 || block_k <= 0) return MI355_EINVAL;
+    // the tiled kernels are built for 128x128 weight blocks; other block sizes run on the plain kernel
+    const bool blocks128 = block_n == kBlockN && block_k == kBlockK;
+    if (!blocks128 && variant != MI355_GEMM_AUTO && variant != MI355_GEMM_GENERIC) return MI355_EUNSUPPORTED;
     if (M == 0 || N == 0) return MI355_OK;
     if (K == 0) return MI355_ESHAPE;
     if (!A || !B || !As || !Bs || !C) return MI355_EINVAL;
@@ -604,7 +607,7 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
                       as_m >= 0 && as_k >= 0;
     const bool was_auto = variant == MI355_GEMM_AUTO;
     if (was_auto) {
-        variant = fast ? pick_variant(M, N, K, cus) : MI355_GEMM_GENERIC;
+        variant = fast && blocks128 ? pick_variant(M, N, K, cus) : MI355_GEMM_GENERIC;
         // stream-K needs its partial-tile slots; without them the plain tile loop gives the same result
         if (variant == MI355_GEMM_TILE256_STREAMK &&
             (!ws || ws_bytes < mi355_block_fp8_gemm_workspace_bytes(M, N, K, variant) || ((uintptr_t)ws & 15)))

@@ -68,8 +68,13 @@ def test_preconditions_are_checked_before_launch():
     assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 256, 96, 1e-10, 4, 1, None) == -2    # K % group
     assert lib.mi355_group_quant_fp8(None, 0, None, None, 4, 256, 128, 1e-10, 2, 1, None) == -1   # null
     assert lib.mi355_group_quant_fp8(None, 0, None, None, 0, 256, 128, 1e-10, 2, 1, None) == 0    # empty
+    # other block sizes: only the plain kernel (AUTO or GENERIC) takes them
     assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 64, 128,
-                                    None, 0, 0, None) == -6
+                                    None, 0, 2, None) == -6
+    assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 64, 128,
+                                    None, 0, 0, None) == -1
+    assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 0, 128,
+                                    None, 0, 0, None) == -1
     assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 4, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 128, 128,
                                     None, 0, 0, None) == -1
     assert lib.mi355_block_fp8_gemm(None, None, None, None, None, 0, 4, 128, 128, 1, 128, 4, 1, 1, 1, 1, 128, 128,

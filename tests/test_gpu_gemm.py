@@ -492,6 +492,40 @@ def test_deepseek_prefill_shapes(hip, N, K, variant):
     _check_full(4096, N, K, variant, seed=N % 97)
 
 
+@pytest.mark.parametrize("bn,bk", [(64, 64), (128, 64), (32, 256), (64, 96)])
+def test_other_block_sizes(hip, bn, bk):
+    """Weight blocks other than 128x128 (the reference kernel takes any block_size, fp8w8a8_block_gemm_kernel.py:100-123):
+    the plain kernel against the C oracle's fp32 per-block order (bit-equal bf16) and the float64 dequant-matmul,
+    with an N tail inside a block and a partial last K block."""
+    from lightllm_amd.quantization import w8a8_block_fp8_matmul
+
+    print(f"gemm block sizes bn={bn} bk={bk}", flush=True)
+    M, N, K = 37, 200, 3 * bk + bk // 2
+    g = H.gen(900 + bn + bk)
+    a = torch.randint(0, 256, (M, K), generator=g, dtype=torch.int32)
+    b = torch.randint(0, 256, (N, K), generator=g, dtype=torch.int32)
+    a[(a & 0x7F) == 0x7F] = 0x38       # no e4m3fn NaN bytes
+    b[(b & 0x7F) == 0x7F] = 0xB8
+    aq = a.to(torch.uint8).cuda().view(torch.float8_e4m3fn)
+    bq = b.to(torch.uint8).cuda().view(torch.float8_e4m3fn)
+    kb, nb = -(-K // bk), -(-N // bn)
+    As = (torch.rand((M, kb), generator=g) * 0.02 + 0.001).cuda()
+    Bs = (torch.rand((nb, kb), generator=g) * 0.02 + 0.001).cuda()
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    w8a8_block_fp8_matmul(aq, bq.t(), As, Bs.t(), C, [bk, bn])
+    torch.cuda.synchronize()
+    want = oracle.block_gemm(tr.bits_of(aq), As.cpu().numpy(), tr.bits_of(bq), Bs.cpu().numpy(), bn=bn, bk=bk)
+    got = C.view(torch.int16).cpu().numpy().view(np.uint16)
+    ref64 = oracle.dequant_matmul_sampled(tr.bits_of(aq), As.cpu().numpy(), tr.bits_of(bq), Bs.cpu().numpy(),
+                                          np.arange(M), np.arange(N), bn=bn, bk=bk)
+    assert np.abs(C.float().cpu().double().numpy() - ref64).max() <= H.GEMM_MAX_REL * np.abs(ref64).max()
+    # same fp32 order per block up to the order inside a block: within one bf16 ulp of the oracle's result
+    wf = tr.bf16_from_bits(want).float()
+    assert (C.float().cpu() - wf).abs().max() <= wf.abs().max() * 2 ** -7
+    with pytest.raises(ValueError):
+        w8a8_block_fp8_matmul(aq, bq.t(), As, Bs.t(), C, [bk, bn], run_config={"variant": "tile128"})
+
+
 def test_generic_strides(hip):
     """B given as a contiguous [K,N] tensor (not the transposed weight view) and row-strided A-scales."""
     from lightllm_amd.quantization import w8a8_block_fp8_matmul
