@@ -346,8 +346,10 @@ def main():
                 w[e], sc[e] = mm_weight_quant(wb)
             return w, sc
 
+        kept = {}
         for (Ng, Kg, tk, mulw, name) in [(4096, 7168, topk, False, "gate_up"), (7168, 2048, 1, True, "down")]:
             w, wscale = expert_weights(Ng, Kg)
+            kept[name] = (w, wscale)
             rows = T if tk == topk else P
             xq, xs = per_token_group_quant_fp8(make_act(rows, Kg, 40, dev), 128)
             out = torch.empty((P, Ng), dtype=torch.bfloat16, device=dev)
@@ -362,6 +364,19 @@ def main():
                            "experts_hit": experts_hit})
             del w, wscale, xq, xs, out
             torch.cuda.empty_cache()
+        # the whole routed-expert FFN of the layer on the same batch: routing tables, quantizer, gate/up GEMM,
+        # fused SiLU-mul + quantizer, down GEMM with the routed weight, sum over the top-k slots
+        from lightllm_amd.fused_moe import fused_experts_impl
+
+        hidden = make_act(T, 7168, 41, dev)
+        (w1, s1), (w2, s2) = kept["gate_up"], kept["down"]
+        us = _time_calls(lambda: fused_experts_impl(hidden, w1, w2, tw, ids, use_fp8_w8a8=True, w1_scale=s1, w2_scale=s2),
+                         3, 2, batches=5)
+        flops = 2.0 * P * (4096 * 7168 + 7168 * 2048)
+        others.append({"name": f"deepseek-v3 routed-expert FFN end to end (fused_experts_impl): {T} tokens, top-{topk} of {E}",
+                       "us": round(us, 1), "TFLOP/s": round(flops / us / 1e6, 1)})
+        del kept, hidden, w1, s1, w2, s2
+        torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "moe":
         # the element-wise steps of the routed-expert FFN at the same size (32768 rows, intermediate 2048,
