@@ -57,17 +57,18 @@ def w8a8_block_fp8_matmul(
     if isinstance(run_config, dict) and "variant" in run_config:
         variant = _VARIANTS[run_config["variant"]]
     lib = _lib.lib()
+    stream = _lib.stream_ptr(A.device)
     ws_ptr, ws_bytes = None, 0
     need = lib.mi355_block_fp8_gemm_workspace_bytes(M, N, K, variant)
     if need:
-        ws = _lib.workspace(A.device, need)
+        ws = _lib.workspace(A.device, need, stream)
         ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
     # the accumulator is cast to the dtype of C, like `accumulator.to(C.dtype.element_ty)` in the reference (:78)
     code = lib.mi355_block_fp8_gemm_dtype(
         A.data_ptr(), B.data_ptr(), Ascale.data_ptr(), Bscale.data_ptr(), C.data_ptr(), M, N, K,
         A.stride(0), B.stride(0), B.stride(1), C.stride(0),
         Ascale.stride(0), Ascale.stride(1), Bscale.stride(0), Bscale.stride(1),
-        block_n, block_k, ws_ptr, ws_bytes, variant, _lib.DTYPE_CODES[C.dtype], _lib.stream_ptr(A.device),
+        block_n, block_k, ws_ptr, ws_bytes, variant, _lib.DTYPE_CODES[C.dtype], stream,
     )
     _lib.check(code, "w8a8_block_fp8_matmul")
     return C
