@@ -269,6 +269,25 @@ def main():
                        "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "rotated_MB": round(4 * Mq * Kq * 2 / 1e6)})
         del sets, nxt
         torch.cuda.empty_cache()
+        # the load-time weight quantizer (bf16 -> e4m3fn + one fp32 scale per 128x128 block) and its inverse on the
+        # gate_up weight; three sources rotate (1.6 GB); each call also allocates its outputs, as the operator does
+        from lightllm_amd.quantization import mm_weight_quant
+        from lightllm_amd.quantization.weight_dequant import weight_dequant
+
+        Nw, Kw = 36864, 7168
+        srcs = [make_act(Nw, Kw, 60 + c, dev) for c in range(3)]
+        nxt = _rotating(srcs)
+        us = _time_calls(lambda: mm_weight_quant(nxt()), 6, 3, batches=5)
+        byts = Nw * Kw * 3 + (Nw // 128) * (Kw // 128) * 4
+        others.append({"name": f"block weight quant [{Nw},{Kw}]", "us": round(us, 1), "GB/s": round(byts / us / 1e3, 1),
+                       "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
+        wq8, ws8 = mm_weight_quant(srcs[0])
+        del srcs, nxt
+        us = _time_calls(lambda: weight_dequant(wq8, ws8), 6, 3, batches=5)
+        others.append({"name": f"block weight dequant [{Nw},{Kw}]", "us": round(us, 1), "GB/s": round(byts / us / 1e3, 1),
+                       "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del wq8, ws8
+        torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "decode":
         # Llama-3-8B decode linears; the weights rotate through enough copies (> 600 MB) that no launch finds them
