@@ -373,9 +373,19 @@ static size_t rows128_workspace(int64_t M, int64_t N, int64_t K, int cus) {
 // against 50.0; Llama-3 down: 27.9 against 30.3) unless K is short (q_b, K = 1536: 21.7 against 17.0).  At 33..64
 // rows it beats the streaming kernels on the large weights (DeepSeek-V3 gate_up, down, o at M = 64: 58.4, 31.7,
 // 31.9 us against 72.3, 42.5, 43.1) and loses on the small ones, where its second launch shows (Llama-3 qkv: 15.0
-// against 13.1); at 32 rows and fewer the streaming kernels are the faster ones.
+// against 13.1); at 32 rows and fewer the streaming kernels are the faster ones but for one case (below).
 static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
-    if (M <= 32 || M > 384) return false;
+    if (M > 384 || M < 16) return false;
+    if (M <= 32) {
+        // 16..32 rows: only where the streaming kernel's 64-row workgroups (two fit a unit) spill into a second,
+        // mostly empty round and this kernel has a well-filled single launch (N = 36864, K = 7168: 576 workgroups on
+        // 512 slots, M = 24 / 32 51.1 / 52.5 us against 46.6 / 46.8 here; on N = 28672, 448 workgroups, the
+        // streaming kernel keeps its lead, 23.8 against 27.4)
+        const int64_t t64 = (N + 63) / 64;
+        const Rows128Plan pl = rows128_plan(M, N, K, cus);
+        return t64 > 2 * (int64_t)cus && t64 <= 3 * (int64_t)cus && pl.splits == 1 && pl.tiles <= cus &&
+               pl.tiles * 20 >= (int64_t)cus * 11;
+    }
     if (M > 256) {
         // 257..384 rows (the activation block of a step is 48 KiB): still ahead where the 128-row tiles are few, K is
         // long and the weights are not small (Llama-3 down at M = 257 / 384: 38.0 / 46.8 us against 66.3 / 66.5;

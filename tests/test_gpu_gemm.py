@@ -304,7 +304,7 @@ def test_rows128_column_major_scales(hip):
 @pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
                                    (128, 2112, 7168), (256, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
                                    (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384), (48, 24576, 1536),
-                                   (64, 28672, 4096)])
+                                   (64, 28672, 4096), (24, 36864, 1024)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
     """Model linears with 33..384 rows that the shape table gives to the weight stream with the activation block in
     LDS."""
