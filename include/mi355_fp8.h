@@ -130,8 +130,9 @@ size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int
  * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as
  * mi355_block_fp8_gemm without the workspace pair: split-K partials and counters go to a fixed array inside the
  * library's device image, MI355_WS_COUNTER_BYTES + MI355_NOALLOC_PARTIAL_MIB MiB per GPU, held from the first call
- * on that GPU until the process ends.  A launch plan that needs more returns MI355_ESCRATCH and launches nothing
- * (mi355_block_fp8_gemm_workspace_bytes() tells the need).  The call allocates and frees nothing; it clears the
+ * on that GPU until the process ends.  A forced variant whose launch plan needs more returns MI355_ESCRATCH and
+ * launches nothing (mi355_block_fp8_gemm_workspace_bytes() tells the need); under MI355_GEMM_AUTO the shape table
+ * falls back to the best plan that fits (fewer or no K splits).  The call allocates and frees nothing; it clears the
  * counter words with a small fill kernel first.  All calls on one GPU share the array: calls that may overlap on
  * one GPU (different streams, concurrently replayed graphs) race - use mi355_block_fp8_gemm with one workspace per
  * stream there. */

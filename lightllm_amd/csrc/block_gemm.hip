@@ -832,7 +832,9 @@ extern "C" int mi355_block_fp8_gemm_noalloc(const void *A, const void *B, const 
                                             int64_t bs_n, int32_t block_n, int32_t block_k, int32_t variant,
                                             void *stream) {
     const size_t need = mi355_block_fp8_gemm_workspace_bytes(M, N, K, variant);
-    if (need > kScratchBytes) return MI355_ESCRATCH;
+    // a forced kernel that needs more than the array holds is an error; the shape table (MI355_GEMM_AUTO) gets
+    // the whole array and takes the next best plan that fits into it
+    if (need > kScratchBytes && variant != MI355_GEMM_AUTO) return MI355_ESCRATCH;
     void *ws = nullptr;
     if (need > 0) {
         ws = scratch_ptr();
