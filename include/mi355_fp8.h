@@ -123,6 +123,11 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
 
 #define MI355_WS_COUNTER_BYTES 65536
 
+/* The kernel MI355_GEMM_AUTO picks for a packed, 16-byte aligned problem of this shape on the CURRENT device (one of
+ * the codes above; MI355_GEMM_GENERIC when K is not a multiple of 128).  No counterpart in the reference, whose
+ * autotuner picks tile sizes at run time (fp8w8a8_block_gemm_kernel.py:120-146); for logs and tests. */
+int32_t mi355_block_fp8_gemm_variant(int64_t M, int64_t N, int64_t K);
+
 /* Bytes of workspace the launch plan of the CURRENT device needs for this shape and variant (0 = none). */
 size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant);
 

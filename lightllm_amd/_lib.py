@@ -23,6 +23,7 @@ SIGNATURES = {
     "mi355_device_info": (_c.c_int, [_c.c_int, _c.POINTER(_i64)]),
     "mi355_group_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _f32, _i64, _i64, _vp]),
     "mi355_block_weight_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp]),
+    "mi355_block_fp8_gemm_variant": (_i32, [_i64, _i64, _i64]),
     "mi355_block_fp8_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "mi355_block_fp8_gemm_noalloc": (
         _c.c_int,

@@ -595,6 +595,14 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     return pl.splits > 1 ? skinny_workspace(M, pl) : 0;
 }
 
+/* The kernel the shape table picks for a packed, aligned problem on the current device (256 compute units when no
+ * device is visible): one of the MI355_GEMM_* codes.  A launch may still fall back when a limit or the workspace of
+ * that kernel is not met. */
+extern "C" int32_t mi355_block_fp8_gemm_variant(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % kBlockK != 0) return MI355_GEMM_GENERIC;
+    return pick_variant(M, N, K, device_cus());
+}
+
 static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, const float *Bs, void *C, int64_t M,
                                int64_t N, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n, int64_t ldc,
                                int64_t as_m, int64_t as_k, int64_t bs_k, int64_t bs_n, int32_t block_n,

@@ -165,3 +165,29 @@ def test_operators_refuse_cpu_tensors():
 
     with pytest.raises(Mi355Error):
         per_token_group_quant_fp8(torch.zeros((2, 128), dtype=torch.bfloat16), 128)
+
+
+def test_shape_table_choices_on_256_compute_units():
+    """The shape -> kernel table for the model linears it was measured on (this container has no GPU: the library
+    plans for 256 compute units).  A change of a rule that moves one of these shapes shows here."""
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    if lib.mi355_device_info(-1, (__import__("ctypes").c_int64 * 8)()) == 0:
+        import pytest
+        pytest.skip("a GPU is visible: the table plans for its own compute-unit count")
+    T256, T128, SKINNY, GENERIC, T256x128, STREAMK, XSHARE, ROWS = 1, 2, 3, 4, 5, 8, 9, 10
+    expect = {
+        (4096, 36864, 7168): T256, (4096, 2112, 7168): T256, (2048, 24576, 1536): T256, (256, 36864, 7168): T256,
+        (512, 36864, 7168): T256,                       # launched as a full round plus a second launch for the rest
+        (1, 28672, 4096): SKINNY, (8, 4096, 14336): SKINNY, (64, 4096, 14336): SKINNY, (8, 36864, 7168): SKINNY,
+        (64, 128256, 4096): XSHARE,
+        (16, 36864, 4096): ROWS, (24, 36864, 7168): ROWS, (64, 28672, 4096): ROWS, (100, 7168, 18432): ROWS, (128, 24576, 1536): ROWS,
+        (128, 2112, 7168): ROWS, (200, 4096, 14336): ROWS, (384, 4096, 14336): ROWS,
+        (300, 36864, 7168): T128, (512, 4096, 4096): T128,
+        (512, 7168, 18432): STREAMK, (2048, 4096, 14336): STREAMK,
+        (1024, 2112, 7168): T256x128,
+        (16, 256, 100): GENERIC,
+    }
+    got = {shape: lib.mi355_block_fp8_gemm_variant(*shape) for shape in expect}
+    assert got == expect, {k: (got[k], expect[k]) for k in expect if got[k] != expect[k]}
