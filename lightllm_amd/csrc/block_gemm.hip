@@ -72,11 +72,29 @@ static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false>(a, grid, st);
 }
 
+#ifndef MI355_SK_PANEL
+#define MI355_SK_PANEL 1
+#endif
+// Runs per tile of the panel split (0 = none): the most that keep tiles * runs within the compute units, with
+// (m tiles * runs) a multiple of the 8 XCDs and at least 12 K steps in a run.
+static int sk_panel_splits(int tiles_m, int tiles_n, int KB, int cus) {
+    int best = 0;
+    for (int s = 2; s <= 32; ++s) {
+        if ((int64_t)tiles_m * tiles_n * s > cus || KB / s < 12) break;
+        if ((tiles_m * s) % 8 == 0) best = s;
+    }
+    return best;
+}
+
 // Stream-K plan of the 256x256 kernel: the number of workgroups (one per compute unit, a multiple of 8), or 0 when
 // the tiles fill whole rounds anyway or there is too little work to give every unit 16 K steps (the 128x128
 // split-K tiles take those shapes).
-static int stream_k_groups(int64_t tiles, int64_t KB, int cus) {
+static int stream_k_groups(int64_t tiles, int64_t KB, int cus, int64_t tiles_m = 0) {
     if (cus < 8 || tiles <= 0) return 0;
+    // a panel split (see launch_pp) stands in for the cut of the unit sequence wherever the shape has one
+    if (MI355_SK_PANEL && tiles_m > 0 && tiles % tiles_m == 0 &&
+        sk_panel_splits((int)tiles_m, (int)(tiles / tiles_m), (int)KB, cus) > 0)
+        return cus / 8 * 8;
     const int64_t units = tiles * KB;
     if (units >= (1ll << 31)) return 0;
     const int64_t groups = cus / 8 * 8;
@@ -87,7 +105,12 @@ static int stream_k_groups(int64_t tiles, int64_t KB, int cus) {
 // Whether the shape table should take that plan.  A workgroup that shares tiles no longer runs in step with the
 // ones that read the same X and W panels, so its K steps are served by the memory side instead of the L2 and take
 // about 2.5 times as long: sharing pays only where the plain loop leaves most of the device idle.
-static bool stream_k_pays(int64_t tiles, int64_t KB, int cus) {
+static bool stream_k_pays(int64_t tiles, int64_t KB, int cus, int64_t tiles_m) {
+    // a panel split that fills three quarters of the device with runs of a long K: measured ahead of every other
+    // kernel from 385 rows on (DeepSeek-V3 down, M = 1024: 128 us against 164 for one workgroup per tile; q_a+kv_a,
+    // M = 2048: 49.6 against 67.9; Llama-3 down, M = 512: 48.8 against 67.8), behind them with K = 4096
+    const int panel = tiles % tiles_m == 0 ? sk_panel_splits((int)tiles_m, (int)(tiles / tiles_m), (int)KB, cus) : 0;
+    if (MI355_SK_PANEL && panel > 0 && KB >= 48 && tiles * panel * 4 >= (int64_t)cus * 3) return true;
     const int groups = stream_k_groups(tiles, KB, cus);
     if (groups == 0) return false;
     const int64_t plain = (tiles + groups - 1) / groups * KB, shared = (tiles * KB + groups - 1) / groups;
@@ -129,6 +152,10 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, int sk_gro
             if (!ws_ok || ws_bytes < stream_k_workspace(sk_groups)) return MI355_EWORKSPACE;
             a.counters = (uint32_t *)ws;
             a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
+            // panel split where the shape allows it: every tile's K range in the same few runs, an XCD working on
+            // one (m tile, run) pair across all n tiles, so that its L2 holds the X rows its workgroups share
+            a.splits = MI355_SK_PANEL ? sk_panel_splits(a.tiles_m, a.tiles_n, a.K / kBlockK, cus) : 0;
+            if (a.splits > 0) sk_groups = a.total_tiles * a.splits;
             const int r = sc4 ? launch_pp_as<false, true, true>(a, sk_groups, lds_bytes, st)
                               : launch_pp_as<false, true, false>(a, sk_groups, lds_bytes, st);
             if (r != MI355_OK) return r;
@@ -507,7 +534,7 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
     const int64_t KB = K / kBlockK;
-    if (M > 128 && stream_k_pays(t256, KB, cus)) return MI355_GEMM_TILE256_STREAMK;
+    if (M > 128 && stream_k_pays(t256, KB, cus, (M + 255) / 256)) return MI355_GEMM_TILE256_STREAMK;
     // 257..384 rows leave the second 256-row tile at most half full; where the 256x256 tiles need a second round
     // anyway the 128x128 ones are ahead (N = 36864, K = 7168, M = 257 / 384: 144 / 148 us against 161 / 165)
     if (M > 256 && M <= 384 && t256 > cus && t128 <= 4 * (int64_t)cus) return MI355_GEMM_TILE128;
@@ -570,7 +597,7 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
         }
     }
     if (variant == MI355_GEMM_TILE256_STREAMK) {
-        const int groups = stream_k_groups(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus);
+        const int groups = stream_k_groups(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus, (M + 255) / 256);
         return groups > 0 ? stream_k_workspace(groups) : (size_t)MI355_WS_COUNTER_BYTES;
     }
     if (variant == MI355_GEMM_TILE128) {
@@ -699,7 +726,7 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
             a.total_tiles = a.tiles_m * a.tiles_n;
             // stream-K when asked for and worth it on this device; the plain tile loop otherwise
             const int groups =
-                variant == MI355_GEMM_TILE256_STREAMK ? stream_k_groups(a.total_tiles, a.K / kBlockK, cus) : 0;
+                variant == MI355_GEMM_TILE256_STREAMK ? stream_k_groups(a.total_tiles, a.K / kBlockK, cus, a.tiles_m) : 0;
             const int r = launch_pp<false>(a, ws, ws_bytes, cus, groups, st);
             if (r != MI355_EUNSUPPORTED) return r;
             return launch_dense<256, 256, 2, 4, 2>(a, st);  // K ranges past the ping-pong kernel's LDS layout

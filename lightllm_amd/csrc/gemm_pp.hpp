@@ -129,9 +129,26 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     const uint32_t lds0 = lds_addr(lds);
     // stream-K: this workgroup's run of (tile, K step) units; workgroups are ranked XCD-major so that one XCD works
     // on neighbouring tiles
-    const uint32_t rank = xcd * per_xcd + in_xcd;
+    uint32_t rank = xcd * per_xcd + in_xcd;
     const uint64_t units = (uint64_t)p.total_tiles * (uint64_t)KB;
-    const uint32_t u_end = SK ? (uint32_t)(((uint64_t)rank + 1u) * units / gridDim.x) : 0u;
+    uint32_t u_end = SK ? (uint32_t)(((uint64_t)rank + 1u) * units / gridDim.x) : 0u;
+    uint32_t u_first = SK ? (uint32_t)((uint64_t)rank * units / gridDim.x) : 0u;
+    if constexpr (SK) {
+        if (p.splits > 0) {
+            // panel split: every tile's K range is cut into p.splits runs; XCD x takes the (m tile, run) pairs
+            // 8*q + x and, of each, all n tiles - so the workgroups of an XCD read the same X rows and K steps at the
+            // same time and its L2 serves all but the first of them.  rank becomes tile * splits + run.
+            const uint32_t q = in_xcd / (uint32_t)p.tiles_n, tn = in_xcd - q * (uint32_t)p.tiles_n;
+            const uint32_t pr = q * 8u + xcd, tm = pr / (uint32_t)p.splits, run = pr - tm * (uint32_t)p.splits;
+            constexpr uint32_t GM = 8;
+            const uint32_t g = tm / GM, first_m = g * GM, gsz = min((uint32_t)p.tiles_m - first_m, GM);
+            const uint32_t id = g * GM * (uint32_t)p.tiles_n + tn * gsz + (tm - first_m);
+            const uint32_t per = (uint32_t)KB / (uint32_t)p.splits, rem = (uint32_t)KB % (uint32_t)p.splits;
+            u_first = id * (uint32_t)KB + run * per + min(run, rem);
+            u_end = u_first + per + (run < rem ? 1u : 0u);
+            rank = id * (uint32_t)p.splits + run;
+        }
+    }
     constexpr uint32_t kNone = 0xffffffffu;
 
     // ---- tile-independent LDS offsets
@@ -350,7 +367,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     uint32_t v_next = persistent ? per_xcd + in_xcd : kNone;  // sequence number of the tile after the current one
     uint32_t v_after = kNone;                                 // and of the one after that (fetched)
     uint32_t fetched = 0;
-    uint32_t v_first = SK ? (uint32_t)((uint64_t)rank * units / gridDim.x) : in_xcd;
+    uint32_t v_first = SK ? u_first : in_xcd;
     if constexpr (ROLES) {
         // a workgroup may enter this loop at any time: all its sequence numbers come from the XCD's queue
         if (tid == 0)
@@ -502,7 +519,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
                 constexpr uint32_t kBlockStride = Cfg::kThreads * 16;  // bytes between a lane's 16x16 blocks
                 const Sc1Buffer xch(p.partials);
                 const uint32_t lane_off = (uint32_t)tid * 16u;
-                const uint32_t mine = (2u * rank + (done.k0 == 0 ? 1u : 0u)) * (uint32_t)Cfg::kPartialBytes + lane_off;
+                const uint32_t mine = (p.splits > 0 ? rank : 2u * rank + (done.k0 == 0 ? 1u : 0u)) * (uint32_t)Cfg::kPartialBytes + lane_off;
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -587,20 +604,31 @@ __global__ __launch_bounds__(512) void streamk_reduce_kernel(const GemmArgs p, u
     const uint32_t id = blockIdx.x / Cfg::TM, i = blockIdx.x % Cfg::TM;
     const uint32_t KB = (uint32_t)(p.K / kBlockK);
     const uint64_t units = (uint64_t)p.total_tiles * KB, t0 = (uint64_t)id * KB;
-    const uint32_t r_lo = (uint32_t)(((t0 + 1u) * groups - 1u) / units);
-    const uint32_t r_hi = (uint32_t)(((t0 + (uint64_t)KB) * groups - 1u) / units);
-    if (r_lo == r_hi) return;
-    // parts in K order: the first rank's run ends inside the tile (its second slot), every later one starts
-    // inside it (its first slot)
+    // slots of the tile's parts in K order.  Runs cut from the unit sequence: the first rank's run ends inside the
+    // tile (its second slot), every later one starts inside it (its first slot).  Panel split: slots
+    // tile * splits + run.
+    uint32_t r_lo, r_hi, first_slot, step;
+    if (p.splits > 0) {
+        r_lo = id * (uint32_t)p.splits;
+        r_hi = r_lo + (uint32_t)p.splits - 1u;
+        first_slot = r_lo;
+        step = 1u;
+    } else {
+        r_lo = (uint32_t)(((t0 + 1u) * groups - 1u) / units);
+        r_hi = (uint32_t)(((t0 + (uint64_t)KB) * groups - 1u) / units);
+        if (r_lo == r_hi) return;
+        first_slot = 2u * r_lo + 1u;
+        step = 2u;
+    }
     const uint8_t *base = (const uint8_t *)p.partials + (uint32_t)tid * 16u + i * TN * kBlockStride;
     v4f acc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-        acc[j] = *(const v4f *)(base + (uint64_t)(2u * r_lo + 1u) * Cfg::kPartialBytes + (uint32_t)j * kBlockStride);
+        acc[j] = *(const v4f *)(base + (uint64_t)first_slot * Cfg::kPartialBytes + (uint32_t)j * kBlockStride);
     for (uint32_t r = r_lo + 1; r <= r_hi; ++r) {
         v4f part[TN];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) part[j] = *(const v4f *)(base + (uint64_t)(2u * r) * Cfg::kPartialBytes + (uint32_t)j * kBlockStride);
+        for (int j = 0; j < TN; ++j) part[j] = *(const v4f *)(base + (uint64_t)(step * r) * Cfg::kPartialBytes + (uint32_t)j * kBlockStride);
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[j] += part[j];
     }

@@ -113,13 +113,17 @@ def test_pingpong_tile_off_grid_k(hip, K):
 # (M, N, K): tiles that do not fill whole rounds of 256 compute units, so that the stream-K plan is taken: one
 # round half empty (DeepSeek q_a+kv_a), a second round one eighth full, few tiles with a long K, ragged edges with
 # a K that is not a multiple of 1024
-STREAM_K_SHAPES = [(4096, 2112, 7168), (512, 36864, 7168), (1024, 7168, 18432), (1000, 8200, 4992), (1000, 2048, 16384)]
+# ... and shapes that take the panel split (every tile's K range in the same runs, one (m tile, run) pair per XCD):
+# even and uneven runs, ragged edges, three runs over eight m tiles
+STREAM_K_SHAPES = [(4096, 2112, 7168), (512, 36864, 7168), (1024, 7168, 18432), (1000, 8200, 4992), (500, 3000, 6400),
+                   (2048, 2112, 7168), (300, 4096, 14336), (1000, 2048, 16384)]
 
 
 @pytest.mark.parametrize("M,N,K", STREAM_K_SHAPES)
 def test_stream_k_launch(hip, M, N, K):
-    """Stream-K: the K steps of all tiles are shared evenly between the compute units and partial tiles are added
-    through the workspace in K order.  Against the torch fp32 dequant-matmul (whole matrix) and the float64 oracle
+    """Stream-K: the K steps of all tiles are shared between the compute units - as one cut of the (tile, step)
+    sequence, or as the panel split where the shape has one - and partial tiles are added through the workspace in K
+    order by a second launch.  Against the torch fp32 dequant-matmul (whole matrix) and the float64 oracle
     (sample); identical bits on repeated launches whoever arrives last; counter words zero afterwards.  The shape
     table itself takes this launch only for the last shape (few tiles, long K)."""
     from lightllm_amd import _lib
