@@ -35,7 +35,10 @@
 //     fp32 accumulators to its own slot of the workspace (two slots per workgroup: a run starts and ends inside at
 //     most one tile each); a second launch (streamk_reduce_kernel) adds the parts of every shared tile in K order
 //     and stores it.  (Adding them in the last workgroup to arrive at a tile was 3 to 8 % slower: one compute unit
-//     reads the parts of a tile at a fraction of the rate the whole device does.)
+//     reads the parts of a tile at a fraction of the rate the whole device does.)  Where the shape allows it the
+//     host asks for a panel split instead (p.splits > 0): every tile's K range in the same p.splits runs and one
+//     (m tile, run) pair per XCD across all n tiles, so that the workgroups of an XCD share their X rows in its L2
+//     - cut as one sequence, neighbouring runs share nothing and the launch is bound by what they all pull.
 //   * ROLES (grouped launch with a workspace): schedule blocks with at most 64 rows are weight streams, and this
 //     tile streams badly (32 KiB of W in flight per step, three quarters of the X area and half of the waves
 //     idle).  They go to the 64 x 512 tile of gemm_small.hpp instead, in the same launch: a split kernel has
