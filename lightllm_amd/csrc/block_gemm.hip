@@ -423,6 +423,11 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         // DeepSeek-V3 down 70.6 / 86.6 against 97.7 / 106.4; Llama-3 qkv 26.0 / 32.0 against 36.3); on 15 MB of
         // weights (q_a+kv_a) it is not (24.1 against 23.5 at M = 320)
         const int64_t tiles = (N + 127) / 128;
+        // from about 340 rows on the 256x256 tiles with a panel split of K overtake it on the large weights
+        // (DeepSeek-V3 down, M = 352 / 384: 79.4 / 78.3 us against 82.9 / 87.5; Llama-3 down stays: 49.7 against 44.8)
+        if (M > 336 && N * K >= 100000000ll &&
+            stream_k_pays(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus, (M + 255) / 256))
+            return false;
         return K / kBlockK >= 16 && N * K >= 20000000ll && tiles * 2 <= cus &&
                tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
     }
