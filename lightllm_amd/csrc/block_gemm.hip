@@ -438,6 +438,10 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         // 40.1 against 46.7; M = 192: 49.2 against 46.8).  With more tiles than units it loses (DeepSeek-V3 gate_up).
         const int64_t tiles = (N + 127) / 128;
         if (K / kBlockK < 16) return false;
+        // from about 200 rows the panel split of the 256x256 tiles is level or ahead on the large weights, its time
+        // flat in M (DeepSeek-V3 down, M = 208 / 240 / 256: 55.1 / 54.9 / 56.9 us against 58.4 / 60.4 / 63.3;
+        // o_proj 53.1 / 52.8 / 58.1 against 54.9 / 57.5 / 57.6)
+        if (M > 200 && N * K >= 100000000ll && stream_k_pays((N + 255) / 256, K / kBlockK, cus, 1)) return false;
         if (tiles * 2 <= cus) return tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
         return M <= 160 && tiles <= cus;
     }

@@ -187,6 +187,7 @@ def test_shape_table_choices_on_256_compute_units():
         (300, 36864, 7168): T128, (512, 4096, 4096): T128,
         (512, 7168, 18432): STREAMK, (2048, 4096, 14336): STREAMK, (1024, 7168, 18432): STREAMK,
         (2048, 2112, 7168): STREAMK, (512, 4096, 14336): STREAMK,     # the panel split
+        (240, 7168, 18432): STREAMK, (352, 7168, 18432): STREAMK, (300, 7168, 18432): ROWS,
         (1024, 2112, 7168): T256x128,
         (16, 256, 100): GENERIC,
     }

@@ -116,7 +116,8 @@ def test_pingpong_tile_off_grid_k(hip, K):
 # ... and shapes that take the panel split (every tile's K range in the same runs, one (m tile, run) pair per XCD):
 # even and uneven runs, ragged edges, three runs over eight m tiles
 STREAM_K_SHAPES = [(4096, 2112, 7168), (512, 36864, 7168), (1024, 7168, 18432), (1000, 8200, 4992), (500, 3000, 6400),
-                   (2048, 2112, 7168), (300, 4096, 14336), (1000, 2048, 16384)]
+                   (2048, 2112, 7168), (300, 4096, 14336), (1000, 2048, 16384), (240, 7168, 18432),
+                   (352, 7168, 16384)]
 
 
 @pytest.mark.parametrize("M,N,K", STREAM_K_SHAPES)
@@ -306,7 +307,7 @@ def test_rows128_column_major_scales(hip):
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
-                                   (128, 2112, 7168), (256, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
+                                   (128, 2112, 7168), (200, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
                                    (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384), (48, 24576, 1536),
                                    (64, 28672, 4096), (24, 36864, 1024)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
