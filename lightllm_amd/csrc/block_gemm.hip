@@ -354,6 +354,7 @@ static int launch_xshare(GemmArgs &a, int splits, void *ws, hipStream_t st) {
 constexpr int kRows128MinSteps = 6;
 
 static int rows128_mt(int64_t M) { return (int)((M + 15) / 16); }
+constexpr int64_t kRows128NarrowMaxM = 208;  // the last row count with narrow workgroups above 128 rows
 
 // Workgroup width, K sharing and tile count of a launch.  Up to 128 rows a workgroup is 8 waves x 32 weight rows;
 // beyond, 8 waves x 16.  While the tiles leave compute units idle the K range is shared, never below
@@ -363,7 +364,7 @@ static int rows128_mt(int64_t M) { return (int)((M + 15) / 16); }
 // tiles (DeepSeek-V3 gate_up, N = 36864: 231 tiles of 160 rows, M = 64 / 128: 50.3 / 62.8 us against 59.4 / 68.8
 // for 144 tiles of 256; q_b, N = 24576, K = 1536: 16.6 against 21.4 with K shared by two).
 struct Rows128Plan {
-    int wv, bn, splits, tiles;
+    int wv, bn, splits, tiles, tn;
 };
 
 static Rows128Plan rows128_plan(int64_t M, int64_t N, int64_t K, int cus) {
@@ -371,6 +372,7 @@ static Rows128Plan rows128_plan(int64_t M, int64_t N, int64_t K, int cus) {
     const int64_t KB = K / kBlockK;
     pl.wv = 8;
     pl.bn = M <= 128 ? 256 : 128;
+    pl.tn = M <= 128 ? 2 : 1;
     if (M <= 128) {
         for (int wv = 5; wv <= 6; ++wv) {
             const int64_t tiles = (N + 32 * wv - 1) / (32 * wv);
@@ -381,6 +383,26 @@ static Rows128Plan rows128_plan(int64_t M, int64_t N, int64_t K, int cus) {
                 pl.tiles = (int)tiles;
                 return pl;
             }
+        }
+    }
+    if (M > 128 && M <= kRows128NarrowMaxM) {
+        // one round of workgroups of just the width that fits it: two 16-row blocks per wave (5..8 waves, 160..256
+        // weight rows) where N is wide enough for that, else one (4..7 waves, 64..112 weight rows)
+        const int64_t wv2 = (N + 32 * (int64_t)cus - 1) / (32 * (int64_t)cus);
+        int64_t wv1 = (N + 16 * (int64_t)cus - 1) / (16 * (int64_t)cus);
+        if (wv1 < 4) wv1 = 4;
+        const int tn = wv2 >= 5 ? 2 : 1;
+        const int64_t wv = tn == 2 ? wv2 : wv1, bn = 16 * tn * wv;
+        const int64_t tiles = (N + bn - 1) / bn;
+        // (four-wave workgroups fall behind the 128x128 tiles a little earlier: N = 16384, K = 7168, M = 208: 63.6 us
+        // against 60.9)
+        if (wv <= (tn == 2 ? 8 : 7) && (wv > 4 || M <= 192) && tiles <= cus && tiles * 20 >= (int64_t)cus * 11) {
+            pl.wv = (int)wv;
+            pl.bn = (int)bn;
+            pl.splits = 1;
+            pl.tiles = (int)tiles;
+            pl.tn = tn;
+            return pl;
         }
     }
     const int64_t tiles = (N + pl.bn - 1) / pl.bn;
@@ -437,13 +459,22 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         // 42.5), and up to 160 rows also where the tiles about fill the device (Llama-3 gate_up, 224 tiles, M = 160:
         // 40.1 against 46.7; M = 192: 49.2 against 46.8).  With more tiles than units it loses (DeepSeek-V3 gate_up).
         const int64_t tiles = (N + 127) / 128;
+        // up to 208 rows a single round of narrower workgroups (160..256 weight rows at two blocks per wave, 64..112
+        // at one) beats the square tiles (N = 36864, K = 7168, M = 144 / 192: 69.1 / 80.5 us against 82.7 / 85.9;
+        // N = 28672, K = 4096: 35.8 / 42.0 against 43.3 / 48.4; q_b, K = 1536: 15.3 / 18.3 against 19.6 / 21.3);
+        // its time grows with M (every wave reads the whole X block from LDS) and the square tiles are level or
+        // ahead from about 220 rows
+        {
+            const Rows128Plan pl = rows128_plan(M, N, K, cus);
+            if (pl.tn == 2 || pl.wv != 8) return true;
+        }
         if (K / kBlockK < 16) return false;
         // from about 200 rows the panel split of the 256x256 tiles is level or ahead on the large weights, its time
         // flat in M (DeepSeek-V3 down, M = 208 / 240 / 256: 55.1 / 54.9 / 56.9 us against 58.4 / 60.4 / 63.3;
         // o_proj 53.1 / 52.8 / 58.1 against 54.9 / 57.5 / 57.6)
         if (M > 200 && N * K >= 100000000ll && stream_k_pays((N + 255) / 256, K / kBlockK, cus, 1)) return false;
         if (tiles * 2 <= cus) return tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
-        return M <= 160 && tiles <= cus;
+        return tiles <= cus && (M <= 160 || (M <= kRows128NarrowMaxM && tiles * 8 >= (int64_t)cus * 7));
     }
     // up to 128 rows: a single well-filled launch always pays (narrow or full-width workgroups on 0.55 cus .. cus
     // tiles with K unshared: DeepSeek-V3 gate_up at M = 64: 49.7 us against 69.9 - 72.5 for the streaming kernels,
@@ -460,16 +491,17 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
 static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t as_m, int64_t as_k, int cus) {
     if (M > 384) return false;
     if (M * lda >= (1ll << 32) || M * as_m * 4 >= (1ll << 32) || as_k * 32 >= (1ll << 32)) return false;
-    const int splits = rows128_splits(M, N, K, cus);
-    const int64_t steps = (K / kBlockK + splits - 1) / splits;
-    if (M > 256) return Rows128Cfg<24, 2, 1>::lds_bytes((int)steps) <= 160 * 1024;
-    if (M > 128) return Rows128Cfg<16, 2, 1>::lds_bytes((int)steps) <= 160 * 1024;
-    return Rows128Cfg<8, 3, 2>::lds_bytes((int)steps) <= 160 * 1024;
+    const Rows128Plan pl = rows128_plan(M, N, K, cus);
+    const int64_t steps = (K / kBlockK + pl.splits - 1) / pl.splits;
+    // Rows128Cfg::lds_bytes for the plan's tile: the ring, the W scales of the tile's n blocks, two X scale chunks
+    const int64_t mt = rows128_mt(M), ns = mt <= 8 ? 3 : 2, nblk = (pl.bn + 2 * kBlockN - 2) / kBlockN;
+    const int64_t ring = ns * (16 * mt * 128 + (int64_t)pl.bn * 128);
+    return ((ring + nblk * steps * 4 + 127) & ~127ll) + 2 * 16 * mt * 32 <= 160 * 1024;
 }
 
-template <int MT, int WV>
+template <int MT, int WV, int TN = (MT <= 8 ? 2 : 1)>
 static int launch_rows128_as(GemmArgs &a, const Rows128Plan &pl, void *ws, hipStream_t st) {
-    constexpr int TN = MT <= 8 ? 2 : 1, NS = MT <= 8 ? 3 : 2;
+    constexpr int NS = MT <= 8 ? 3 : 2;
     using Cfg = Rows128Cfg<MT, NS, TN, WV>;
     const int KB = a.K / kBlockK;
     const int steps = (KB + pl.splits - 1) / pl.splits;
@@ -480,7 +512,7 @@ static int launch_rows128_as(GemmArgs &a, const Rows128Plan &pl, void *ws, hipSt
         if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
         return launch(kernel, dim3(pl.tiles), dim3(Cfg::kThreads), lds_bytes, st, a);
     }
-    if constexpr (WV == 8) {
+    if constexpr (WV == 8 && TN == (MT <= 8 ? 2 : 1)) {
         constexpr auto kernel = block_fp8_gemm_rows128_kernel<MT, NS, TN, 8, true>;
         if (!allow_lds<kernel>(160 * 1024)) return MI355_ELAUNCH;
         a.splits = pl.splits;
@@ -497,6 +529,23 @@ static int launch_rows128(GemmArgs &a, const Rows128Plan &pl, void *ws, hipStrea
     if constexpr (MT <= 8) {
         if (pl.wv == 5) return launch_rows128_as<MT, 5>(a, pl, ws, st);
         if (pl.wv == 6) return launch_rows128_as<MT, 6>(a, pl, ws, st);
+    } else if constexpr (MT <= (kRows128NarrowMaxM + 15) / 16) {
+        if (pl.tn == 2) {
+            switch (pl.wv) {
+            case 5: return launch_rows128_as<MT, 5, 2>(a, pl, ws, st);
+            case 6: return launch_rows128_as<MT, 6, 2>(a, pl, ws, st);
+            case 7: return launch_rows128_as<MT, 7, 2>(a, pl, ws, st);
+            case 8: return launch_rows128_as<MT, 8, 2>(a, pl, ws, st);
+            default: return MI355_EINVAL;
+            }
+        }
+        switch (pl.wv) {
+        case 4: return launch_rows128_as<MT, 4>(a, pl, ws, st);
+        case 5: return launch_rows128_as<MT, 5>(a, pl, ws, st);
+        case 6: return launch_rows128_as<MT, 6>(a, pl, ws, st);
+        case 7: return launch_rows128_as<MT, 7>(a, pl, ws, st);
+        default: break;
+        }
     }
     return launch_rows128_as<MT, 8>(a, pl, ws, st);
 }
@@ -524,7 +573,11 @@ static size_t tile256x128_workspace(int64_t M, int64_t N, int splits) {
 // The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
 //   129 <= M <= 384, K >= 2048, at most cus/2 tiles
 //     of 128 weight rows (cus if M <= 160; above
-//     256 rows only if N*K >= 2e7)                   the weight stream with the activation block in LDS
+//     256 rows only if N*K >= 2e7; 201..256 and
+//     337..384 rows on N*K >= 1e8 go to the panel
+//     split of stream-K instead)                     the weight stream with the activation block in LDS
+//   129 <= M <= 208 (192), 0.55 cus .. cus tiles of
+//     160..256 or of 80..112 (64) weight rows         the same, workgroups of that width, K unshared
 //   65 <= M <= 128, K >= 2048                        the same with 256 weight rows per workgroup
 //   33 <= M <= 64, N*K >= 1e8, at most cus tiles     the same, unless the kernel below would run
 //   33 <= M <= 128, 0.55 cus .. cus tiles of 160,

@@ -6,7 +6,8 @@
 // (gemm_small.hpp) with more rows and a dense epilogue:
 //
 //   16*MT activation rows (MT MFMA row blocks) x 128*TN weight rows, K step 128.
-//     TN = 2: up to 128 rows (MT <= 8) against 256 weight rows; TN = 1: up to 384 rows (MT <= 24) against 128.
+//     TN = 2: up to 128 rows (MT <= 8; 16 on two ring slots) against 256 weight rows; TN = 1: up to 384 rows
+//     (MT <= 24) against 128.
 //   WV waves (8; fewer for some unsplit launches, see below), wave w owns 16*TN weight rows and all activation rows:
 //   MT x TN MFMA blocks per K step (the X operand blocks are read from LDS eight at a time).
 //   NS ring slots of { X 16*MT x 128 B, W 128*TN x 128 B }.  A wave fetches its own W rows (2*TN requests of 1 KiB
@@ -23,6 +24,10 @@
 //   What a unit pulls is X and W together - the X block comes from L2, but through the same requests - so a launch
 //   whose 256-row tiles leave units idle and whose K cannot be shared usefully runs narrower workgroups instead
 //   (WV = 5 or 6: 160 or 192 weight rows), as many as there are units: every unit then loads less per K step.
+//   The same holds for 129..208 rows on a wide N, whose 128-row tiles need a second round and whose 256x256 tiles
+//   leave units idle: workgroups of 4..7 waves at TN = 1 (64..112 weight rows) or, on a wider N still, 5..8 waves at
+//   TN = 2 with up to 13 row blocks (160..256 weight rows), whichever makes one round.  Every wave reads the whole X
+//   block from LDS, so the time of such a launch grows with M and the square tiles take over from about 220 rows.
 //
 //   (Half-width tiles of four waves on two slots, two workgroups to a unit, were tried for shapes whose 256-row
 //   tiles leave units idle and cannot share K usefully - N = 36864: 144 tiles on 256 units - and were slower: 85 us
@@ -36,7 +41,7 @@ namespace mi355 {
 
 template <int MT, int NS, int TN_ = 2, int WV = 8>
 struct Rows128Cfg {
-    static_assert(WV >= 4 && WV <= 8 && MT >= 1 && MT <= (TN_ == 2 ? 8 : 24) && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
+    static_assert(WV >= 4 && WV <= 8 && MT >= 1 && MT <= (TN_ == 2 ? 16 : 24) && (NS == 2 || NS == 3) && (TN_ == 1 || TN_ == 2), "");
     static constexpr int TN = TN_, WNS = 16 * TN, kWaves = WV, kThreads = 64 * WV, BN = WNS * WV;
     static constexpr int NBLK = (BN + 2 * kBlockN - 2) / kBlockN;  // 128-wide n blocks a tile can touch
     static constexpr int NWW = 2 * TN;                         // W requests per wave and step (8 rows each)

@@ -255,7 +255,7 @@ def test_shared_activation_stream_kernel(hip):
 
 def test_rows128_stream_kernel(hip):
     """The weight stream with the activation block in LDS (M <= 384; 256 weight rows per workgroup up to 128 rows,
-    128 beyond): random shapes - every row-block
+    128 beyond, other widths where they make a single round): random shapes - every row-block
     count, N tails that cut a wave's rows, a workgroup's rows and the vector stores, K from one step (fewer
     steps than ring slots) to 144 so that whole-K and shared-K launches (second launch adds the partial sums) both
     occur - against the torch fp32 dequant-matmul, the float64 oracle on a sample and the 128x128 tile (same
@@ -269,7 +269,11 @@ def test_rows128_stream_kernel(hip):
                int(rng.choice([128, 256, 640, 1024, 2048, 7168, 18432]))) for _ in range(18)]
     cases += [(128, 256, 128), (65, 4096, 14336), (127, 2112, 7168), (80, 520, 2304), (256, 128, 128), (129, 7168, 2048),
               (100, 160 * 200 + 8, 640), (40, 192 * 230 - 3, 512), (128, 160 * 141, 256),   # 160- and 192-row workgroups
-              (255, 2112, 7168), (144, 1000, 4096), (384, 640, 4096), (257, 136, 256), (383, 4100, 2048)]
+              (255, 2112, 7168), (144, 1000, 4096), (384, 640, 4096), (257, 136, 256), (383, 4100, 2048),
+              # 129..208 rows, one round of 64- to 112-row workgroups (one 16-row block per wave) ...
+              (130, 9100, 384), (192, 16384 - 7, 256), (208, 20000, 640), (150, 24576 - 1, 128), (176, 28672 - 20, 256),
+              # ... or of 160- to 256-row ones (two blocks per wave) where N is wider
+              (144, 36864 - 5, 256), (208, 45000, 128), (160, 52003, 256), (199, 65536 - 9, 128)]
     shared = 0
     for case, (M, N, K) in enumerate(cases):
         print(f"gemm rows128 case {case}: M={M} N={N} K={K}", flush=True)
@@ -308,6 +312,7 @@ def test_rows128_column_major_scales(hip):
 
 @pytest.mark.parametrize("M,N,K", [(128, 36864, 7168), (100, 7168, 18432), (64, 7168, 16384), (65, 4096, 14336),
                                    (128, 2112, 7168), (200, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
+                                   (192, 36864, 7168), (208, 24576, 1536),
                                    (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384), (48, 24576, 1536),
                                    (64, 28672, 4096), (24, 36864, 1024)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
