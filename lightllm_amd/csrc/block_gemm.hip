@@ -570,6 +570,8 @@ static size_t tile256x128_workspace(int64_t M, int64_t N, int splits) {
     return (size_t)MI355_WS_COUNTER_BYTES + (size_t)tiles * splits * 256 * 128 * 4;
 }
 
+static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus);
+
 // The shape -> kernel table (measured on the DeepSeek-V3 and Llama-3 linears over M = 128..4096):
 //   129 <= M <= 384, K >= 2048, at most cus/2 tiles
 //     of 128 weight rows (cus if M <= 160; above
@@ -598,8 +600,10 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     const int64_t KB = K / kBlockK;
     if (M > 128 && stream_k_pays(t256, KB, cus, (M + 255) / 256)) return MI355_GEMM_TILE256_STREAMK;
     // 257..384 rows leave the second 256-row tile at most half full; where the 256x256 tiles need a second round
-    // anyway the 128x128 ones are ahead (N = 36864, K = 7168, M = 257 / 384: 144 / 148 us against 161 / 165)
-    if (M > 256 && M <= 384 && t256 > cus && t128 <= 4 * (int64_t)cus) return MI355_GEMM_TILE128;
+    // anyway the 128x128 ones are ahead (N = 36864, K = 7168, M = 257 / 384: 144 / 148 us against 161 / 165) -
+    // unless the second round is small enough to run as a launch of its own (130 / 139 us then)
+    if (M > 256 && M <= 384 && t256 > cus && t128 <= 4 * (int64_t)cus && n_split_rows(M, N, K, cus) == 0)
+        return MI355_GEMM_TILE128;
     if (t128 <= 2 * (int64_t)cus && (t256 < (int64_t)cus * 3 / 8 || KB <= 64)) {
         // a narrow N under many rows: 256x128 tiles with K shared load half as much X per product as the 128x128
         // ones and still fill the device (q_a+kv_a, N = 2112, K = 7168, M = 768 / 1024 / 1536: 35.0 / 40.6 / 50.6 us

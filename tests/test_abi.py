@@ -185,7 +185,8 @@ def test_shape_table_choices_on_256_compute_units():
         (16, 36864, 4096): ROWS, (24, 36864, 7168): ROWS, (64, 28672, 4096): ROWS, (100, 7168, 18432): ROWS, (128, 24576, 1536): ROWS,
         (128, 2112, 7168): ROWS, (200, 4096, 14336): ROWS, (384, 4096, 14336): ROWS,
         (192, 36864, 7168): ROWS, (176, 28672, 4096): ROWS, (224, 28672, 4096): T128,   # narrower workgroups up to 208 rows
-        (300, 36864, 7168): T128, (512, 4096, 4096): T128,
+        (300, 28672, 4096): T256, (512, 4096, 4096): T128,
+        (300, 36864, 7168): T256,                       # likewise: a full round and the rest
         (512, 7168, 18432): STREAMK, (2048, 4096, 14336): STREAMK, (1024, 7168, 18432): STREAMK,
         (2048, 2112, 7168): STREAMK, (512, 4096, 14336): STREAMK,     # the panel split
         (240, 7168, 18432): STREAMK, (352, 7168, 18432): STREAMK, (300, 7168, 18432): ROWS,

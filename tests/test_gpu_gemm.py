@@ -407,7 +407,7 @@ def test_256x128_tiles_with_shared_k(hip, M, N, K):
     assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
 
 
-@pytest.mark.parametrize("M,N,K", [(512, 36864, 1024), (400, 36864 + 72, 2048), (768, 24576, 1536)])
+@pytest.mark.parametrize("M,N,K", [(512, 36864, 1024), (400, 36864 + 72, 2048), (768, 24576, 1536), (300, 36864, 2048)])
 def test_rest_of_a_round_runs_as_its_own_launch(hip, M, N, K):
     """256x256 tiles that fill the device once and leave a small rest: the table runs the rest (the last weight
     rows) as a second launch with the kernel its own shape gets.  Same products in the same order per output as
