@@ -634,14 +634,16 @@ static size_t tile128_workspace(int64_t M, int64_t N, int splits) {
 // A launch of 256x256 tiles that fills the device once and leaves a small rest for a second round runs the rest
 // as a launch of its own, with whatever the table gives its shape (mostly 128x128 tiles, which spread it over the
 // whole device): N = 36864, K = 7168, M = 512 (288 tiles on 256 units) 137 us against 169; q_b, M = 768, 43.6
-// against 50.2.  With two or more full rounds, or a rest of more than half a round, it gains nothing.  Returns the
-// number of weight rows of the first launch, 0 for no split.
+// against 50.2.  After two full rounds a rest of up to a quarter round still gains a little (M = 1024, 576 tiles:
+// 248 us against 260; q_b, M = 1536: 77.8 against 83.3); with more rounds or a larger rest it gains nothing (3.5
+// rounds: 235 against 220).  Returns the number of weight rows of the first launch, 0 for no split.
 static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus) {
     (void)K;
     const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256, t256 = tiles_m * tiles_n;
-    if (tiles_m > cus || t256 <= cus || t256 >= 2 * (int64_t)cus) return 0;
-    if ((t256 - cus) * 2 > cus) return 0;
-    const int64_t n1 = (int64_t)cus / tiles_m * 256;
+    const int64_t rounds = t256 / cus, rest = t256 - rounds * cus;
+    if (tiles_m > cus || rounds < 1 || rounds > 2 || rest == 0) return 0;
+    if (rest * 2 * rounds > cus) return 0;
+    const int64_t n1 = rounds * (int64_t)cus / tiles_m * 256;
     return n1 > 0 && n1 < N ? n1 : 0;
 }
 

@@ -407,9 +407,10 @@ def test_256x128_tiles_with_shared_k(hip, M, N, K):
     assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
 
 
-@pytest.mark.parametrize("M,N,K", [(512, 36864, 1024), (400, 36864 + 72, 2048), (768, 24576, 1536), (300, 36864, 2048)])
+@pytest.mark.parametrize("M,N,K", [(512, 36864, 1024), (400, 36864 + 72, 2048), (768, 24576, 1536), (300, 36864, 2048),
+                                   (1024, 36864, 1024)])
 def test_rest_of_a_round_runs_as_its_own_launch(hip, M, N, K):
-    """256x256 tiles that fill the device once and leave a small rest: the table runs the rest (the last weight
+    """256x256 tiles that fill the device once (or twice) and leave a small rest: the table runs the rest (the last weight
     rows) as a second launch with the kernel its own shape gets.  Same products in the same order per output as
     the one-launch 256x256 tiles when that kernel does not share K, close to it otherwise; fp32 reference and
     float64 oracle as everywhere."""
@@ -418,7 +419,8 @@ def test_rest_of_a_round_runs_as_its_own_launch(hip, M, N, K):
     print(f"gemm rest-of-a-round split M={M} N={N} K={K}", flush=True)
     cus = _lib.device_info()["compute_units"]
     t256 = -(-M // 256) * -(-N // 256)
-    if not (cus < t256 <= cus * 3 // 2):
+    rounds, rest = divmod(t256, cus)
+    if not (rounds in (1, 2) and 0 < rest * 2 * rounds <= cus):
         pytest.skip("shape chosen for 256 compute units")
     xq, xs, wq, ws = _prep(M, N, K, seed=M + K)
     c = _run(xq, xs, wq, ws, None).clone()
