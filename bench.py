@@ -322,7 +322,7 @@ def main():
         for (Np, Kp, name) in shapes:
             wq, ws = make_weight(Np, Kp, 30, dev)
             wq_t, ws_t = wq.t(), ws.t()
-            for Mp in (128, 256, 512, 1024, 2048, 4096):
+            for Mp in (128, 192, 256, 512, 1024, 2048, 4096):
                 if name == "gate_up" and Mp == 4096:
                     continue  # the headline
                 xq, xs = per_token_group_quant_fp8(make_act(Mp, Kp, 31, dev), 128)
