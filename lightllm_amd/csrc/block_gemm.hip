@@ -482,10 +482,21 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
     const Rows128Plan pl = rows128_plan(M, N, K, cus);
     if (pl.splits == 1 && pl.tiles <= cus && pl.tiles * 20 >= (int64_t)cus * 11) return true;
     if (M > 64) return K / kBlockK >= 16;
-    // 33..64 rows with K shared or more tiles than units: on the large weights only, and not where the
+    // 33..64 rows with K shared or more tiles than units: on the large weights, and not where the
     // shared-activation streaming kernel runs (lm_head, N = 128256, K = 4096, M = 64: 116 us against 110 - its small
     // workgroups fill the second round better)
-    return N * K >= 100000000ll && pl.tiles <= cus && !xshare_pays(M, N, K, cus);
+    if (pl.tiles > cus || xshare_pays(M, N, K, cus)) return false;
+    // ... unless the streaming kernel's workgroups come out as one per unit with K whole (N = 16384, K = 7168,
+    // M = 64: 25.9 us against 29.9) ...
+    const SkinnyPlan sp = skinny_plan(M, N, K, cus);
+    const int64_t wgs = (int64_t)sp.tiles * sp.splits;
+    if (N * K >= 100000000ll) return !(sp.splits == 1 && wgs == cus);
+    // ... and on the mid-size ones (from 40 MB) where they come out as neither one nor two per unit: N = 10240,
+    // K = 8192 (640 of them), M = 64: 24.5 us against 33.6; 14336 x 4096 (896): 19.6 against 24.0; 12288 x 4096 (768):
+    // 18.0 against 22.4; 5120 x 13824 (640): 21.4 against 28.8.  With 512 or 256 of them it keeps its lead (8192 x
+    // 8192: 21.3 against 22.9; 16384 x 4096: 18.7 against 21.3), and on smaller weights the second launch shows
+    // (6144 x 4096: 12.8 against 14.6).
+    return N * K >= 40000000ll && wgs != cus && wgs != 2 * (int64_t)cus;
 }
 
 static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t as_m, int64_t as_k, int cus) {
@@ -581,7 +592,9 @@ static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus);
 //   129 <= M <= 208 (192), 0.55 cus .. cus tiles of
 //     160..256 or of 80..112 (64) weight rows         the same, workgroups of that width, K unshared
 //   65 <= M <= 128, K >= 2048                        the same with 256 weight rows per workgroup
-//   33 <= M <= 64, N*K >= 1e8, at most cus tiles     the same, unless the kernel below would run
+//   33 <= M <= 64, at most cus tiles, N*K >= 1e8 or
+//     (N*K >= 4e7 and the streaming kernel's
+//     workgroups neither cus nor 2 cus)              the same, unless the kernel below would run
 //   33 <= M <= 128, 0.55 cus .. cus tiles of 160,
 //     192 or 256 weight rows with K unshared          the same, workgroups of that width
 //   M <= 64                                          weight streaming (M > 32 and N/128 about the unit count: the
