@@ -106,11 +106,12 @@ static int stream_k_groups(int64_t tiles, int64_t KB, int cus, int64_t tiles_m =
 // ones that read the same X and W panels, so its K steps are served by the memory side instead of the L2 and take
 // about 2.5 times as long: sharing pays only where the plain loop leaves most of the device idle.
 static bool stream_k_pays(int64_t tiles, int64_t KB, int cus, int64_t tiles_m) {
-    // a panel split that fills three quarters of the device with runs of a long K: measured ahead of every other
+    // a panel split that fills three eighths of the device with runs of a long K: measured ahead of every other
     // kernel from 385 rows on (DeepSeek-V3 down, M = 1024: 128 us against 164 for one workgroup per tile; q_a+kv_a,
-    // M = 2048: 49.6 against 67.9; Llama-3 down, M = 512: 48.8 against 67.8), behind them with K = 4096
+    // M = 2048: 49.6 against 67.9; Llama-3 down, M = 512: 48.8 against 67.8; N = 4096, K = 7168, M = 512, 128
+    // workgroups: 34.5 against 39.8; N = 5120, K = 5120, M = 1024: 47.0 against 53.8), behind them with K = 4096
     const int panel = tiles % tiles_m == 0 ? sk_panel_splits((int)tiles_m, (int)(tiles / tiles_m), (int)KB, cus) : 0;
-    if (MI355_SK_PANEL && panel > 0 && KB >= 48 && tiles * panel * 4 >= (int64_t)cus * 3) return true;
+    if (MI355_SK_PANEL && panel > 0 && KB >= 40 && tiles * panel * 8 >= (int64_t)cus * 3) return true;
     const int groups = stream_k_groups(tiles, KB, cus);
     if (groups == 0) return false;
     const int64_t plain = (tiles + groups - 1) / groups * KB, shared = (tiles * KB + groups - 1) / groups;
@@ -625,7 +626,12 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
         // a narrow N under many rows: 256x128 tiles with K shared load half as much X per product as the 128x128
         // ones and still fill the device (q_a+kv_a, N = 2112, K = 7168, M = 768 / 1024 / 1536: 35.0 / 40.6 / 50.6 us
         // against 38.7 / 60.2 / 60.6)
-        if (M >= 768 && (N + 127) / 128 <= 24 && tile256x128_splits(M, N, K, cus) >= 2) return MI355_GEMM_TILE256x128;
+        // ... and, from two 256-row tiles on, a wider N under a long K (N = 5120, K = 5120, M = 400 / 512: 35.4 /
+        // 37.6 us against 44.7 / 45.1; N = 4096, K = 7168, M = 640: 54.6 against 60.3; on N = 1536 the 128x128 tiles
+        // keep their lead, 21.8 against 25.2, and with K = 4096 too)
+        if (((M >= 768 && (N + 127) / 128 <= 24) || (M > 384 && KB >= 40 && (N + 127) / 128 >= 20)) &&
+            tile256x128_splits(M, N, K, cus) >= 2)
+            return MI355_GEMM_TILE256x128;
         return MI355_GEMM_TILE128;
     }
     if (t256 >= (int64_t)cus * 3 / 8) return MI355_GEMM_TILE256;
@@ -827,8 +833,10 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
             a.total_tiles = a.tiles_m * a.tiles_n;
             a.splits = splits;
             a.counters = (uint32_t *)ws;
-            a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
-            return launch_tile<256, 128, 2, 4, 3, kSplitK>(a, a.total_tiles * splits, st);
+            a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);  // the counter words stay untouched
+            const int r = launch_tile<256, 128, 2, 4, 3, kSplitK>(a, a.total_tiles * splits, st);
+            if (r != MI355_OK) return r;
+            return launch(tile_splitk_reduce_kernel<256, 128, 2, 4>, dim3(a.total_tiles * 16), dim3(512), 0, st, a);
         }
         case MI355_GEMM_TILE128: {
             const int splits = tile128_splits(M, N, K, cus);
@@ -840,7 +848,9 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
             a.splits = splits;
             a.counters = (uint32_t *)ws;
             a.partials = (float *)((uint8_t *)ws + MI355_WS_COUNTER_BYTES);
-            return launch_tile<128, 128, 2, 2, 2, kSplitK>(a, a.total_tiles * splits, st);
+            const int r = launch_tile<128, 128, 2, 2, 2, kSplitK>(a, a.total_tiles * splits, st);
+            if (r != MI355_OK) return r;
+            return launch(tile_splitk_reduce_kernel<128, 128, 2, 2>, dim3(a.total_tiles * 16), dim3(256), 0, st, a);
         }
         case MI355_GEMM_SKINNY_XSHARE: {
             if (M <= 32 || M > 64) return MI355_EUNSUPPORTED;

@@ -29,9 +29,9 @@
 //
 // Launch modes
 //   kDense     one CTA per output tile, whole K, ring.
-//   kSplitK    grid = tiles x splits; each CTA accumulates a K range, stores its fp32 partial to the
-//              workspace in register order, and the CTA that arrives last at the tile's counter adds the
-//              partials in split order (deterministic), writes bf16 and re-zeroes the counter.
+//   kSplitK    grid = tiles x splits; each CTA accumulates a K range and stores its fp32 partial to the
+//              workspace in register order; a second launch (tile_splitk_reduce_kernel) adds the partials in
+//              split order (deterministic) and writes C.
 //   kGrouped   rows are gathered through expert_to_token_index, the tile list is the moe_align2 table, the
 //              weight and its scales are offset by the expert, rows are scattered back on store.
 #pragma once
@@ -367,58 +367,18 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     }
 
 
-    // ---- split-K: publish the partial, let the last CTA of the tile reduce
-    // Partials are exchanged with sc1 accesses and the arrival counter with an agent-scope relaxed atomic: such
-    // stores write through, and such loads read past, the per-XCD L2, so no cache-wide write-back / invalidate
-    // fence is needed (one of those per CTA costs more than the whole GEMM at decode sizes).  Order is kept by
-    // "all my stores acknowledged (vmcnt 0) -> barrier -> one atomic add" on the writer side and
-    // "atomic add returned -> barrier -> loads" on the reader side.  What this relies on: a gfx950 store with
-    // sc1 is complete (vmcnt) only once it has reached the memory side that all XCDs share, and a load with sc1
-    // is served from there, never from a line the reader's own L2 or L1 held before.
+    // ---- split-K: the partial sums go to the workspace in register order ([split][block][thread] float4);
+    // tile_splitk_reduce_kernel, a second launch, adds them in split order and writes C.  (The last workgroup of a
+    // tile adding them alone - one compute unit reads about 40 GB/s - cost more than the launch: 128 KiB partials of
+    // seven splits took 22 us.)
     if constexpr (MODE == kSplitK) {
         constexpr int kTileElems = BM * BN;
-        constexpr int NB = TM * TN;  // 16x16 blocks per lane, 16 bytes each
-        const float *tile_base = p.partials + (int64_t)tile_id * p.splits * kTileElems;
-        const Sc1Buffer xch(tile_base);
-        const uint32_t lane_off = (uint32_t)tid * 16u;
-        {
-            const uint32_t mine = split * (uint32_t)(kTileElems * 4) + lane_off;
+        float *mine = p.partials + ((int64_t)tile_id * p.splits + split) * kTileElems + tid * 4;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) xch.store(mine + (uint32_t)((i * TN + j) * Cfg::kThreads * 16), acc[i][j]);
-        }
-        wait_vmcnt<0>();
-        __syncthreads();
-        // (the arrival word lives in the dynamic allocation: a static __shared__ object would push static +
-        // opt-in dynamic LDS past the 160 KiB a workgroup may ask for)
-        volatile uint32_t *arrived = (volatile uint32_t *)(lds + Cfg::kWsOff + Cfg::NBC * KB * 4);
-        if (tid == 0)
-            *arrived = __hip_atomic_fetch_add(p.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if (*arrived != (uint32_t)p.splits - 1u) return;
-        // the last workgroup adds the partials in split order; the loads of one split are in flight while the
-        // previous one is added (one memory round trip per split, not one per 16 bytes)
-        auto fetch = [&](v4f (&dst)[NB], int sp) {
-            const uint32_t src = (uint32_t)sp * (uint32_t)(kTileElems * 4) + lane_off;
-#pragma unroll
-            for (int b = 0; b < NB; ++b) dst[b] = xch.load(src + (uint32_t)(b * Cfg::kThreads * 16));
-        };
-        auto add = [&](const v4f (&src)[NB], bool first) {
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = first ? src[i * TN + j] : acc[i][j] + src[i * TN + j];
-        };
-        v4f even[NB], odd[NB];
-        fetch(even, 0);
-        for (int sp = 0; sp < p.splits; sp += 2) {
-            if (sp + 1 < p.splits) fetch(odd, sp + 1);
-            add(even, sp == 0);
-            if (sp + 2 < p.splits) fetch(even, sp + 2);
-            if (sp + 1 < p.splits) add(odd, false);
-        }
-        if (tid == 0) __hip_atomic_store(p.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int j = 0; j < TN; ++j) *(v4f *)(mine + (i * TN + j) * Cfg::kThreads * 4) = acc[i][j];
+        return;
     }
 
     // ---- epilogue: lane (r16, g4) holds, for each tm, row m = wave_m*WMS + 16*tm + r16 and, for each MFMA block
@@ -459,6 +419,43 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
                 if (nbase + c < p.N) cp[c] = (uint16_t)out_bits(o[e], p.out_f16);
             }
         }
+    }
+}
+
+// Second launch of a split-K GEMM on the ring tiles: workgroup (tile, block b) - the thread layout of the GEMM's
+// workgroup - adds block b of the tile's partial sums over the splits in split order and stores the 4 outputs of
+// each thread.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN * 64) void tile_splitk_reduce_kernel(const GemmArgs p) {
+    using Cfg = TileCfg<BM, BN, WM, WN, 2>;
+    constexpr int TN = Cfg::TN, NB = Cfg::TM * Cfg::TN, kTileElems = BM * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WN, wave_n = wave % WN;
+    const int r16 = lane & 15, g4 = lane >> 4;
+    const uint32_t tile_id = blockIdx.x / NB, b = blockIdx.x - tile_id * NB;
+    const uint32_t tile_m = tile_id % (uint32_t)p.tiles_m, tile_n = tile_id / (uint32_t)p.tiles_m;
+    const int i = (int)b / TN, j = (int)b % TN;
+    const float *src = p.partials + (int64_t)tile_id * p.splits * kTileElems + (int64_t)b * Cfg::kThreads * 4 + tid * 4;
+    v4f a = *(const v4f *)src;
+    int sp = 1;
+    for (; sp + 4 <= p.splits; sp += 4) {
+        v4f t[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) t[d] = *(const v4f *)(src + (int64_t)(sp + d) * kTileElems);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) a += t[d];
+    }
+    for (; sp < p.splits; ++sp) a += *(const v4f *)(src + (int64_t)sp * kTileElems);
+    const int row = (int)tile_m * BM + wave_m * Cfg::WMS + 16 * i + r16;
+    const int col = (int)tile_n * BN + wave_n * Cfg::WNS + lane_col<TN>(g4, j);
+    if (row >= p.M) return;
+    uint16_t *cp = p.C + (int64_t)row * p.ldc + col;
+    if (p.vec_store && col + 4 <= p.N) {
+        *(v2i *)cp = v2i{(int)pack_out2(a[0], a[1], p.out_f16), (int)pack_out2(a[2], a[3], p.out_f16)};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (col + e < p.N) cp[e] = (uint16_t)out_bits(a[e], p.out_f16);
     }
 }
 

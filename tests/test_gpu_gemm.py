@@ -395,7 +395,7 @@ def test_256x128_tiles_with_shared_k(hip, M, N, K):
     xq, xs, wq, ws = _prep(M, N, K, seed=M + K)
     C1 = _run(xq, xs, wq, ws, "tile256x128").clone()
     assert torch.equal(C1, _run(xq, xs, wq, ws, "tile256x128"))
-    if M >= 768:
+    if M == 768:
         assert torch.equal(C1, _run(xq, xs, wq, ws, None))
     ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
     cos, rel = H.gemm_metrics(C1.float(), ref)
