@@ -1001,8 +1001,31 @@ extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts,
     // one from about 12 rows per expert on (256 experts, top-8, N=4096 K=7168: 512 tokens 1275 us against 1291 for
     // 32-row blocks, 1024 tokens 1314 against 1500, 2048 tokens 1421 against 1885; the same within 1 % at 384
     // tokens).  With fewer rows the 16-row tiles stream the weights at 6.0 TB/s and nothing beats them.
-    const bool two_queues = (int64_t)num_experts * ((N + 255) / 256) > device_cus();
-    if (avg > 64 || (two_queues && avg >= 12)) return 256;
+    const int cus = device_cus();
+    const int64_t tiles256 = (int64_t)num_experts * ((N + 255) / 256);
+    const bool two_queues = tiles256 > cus;
+    // Measured over Qwen3-MoE (128 experts), DeepSeek-V2-Lite (64), Mixtral (8), a DeepSeek-V3 expert-parallel slice
+    // (32 experts, N = 512) and a 16-expert shape, 8 to 8192 tokens, uniform routing:
+    //  * 128-row blocks are ahead of the 256-row launch up to a few hundred rows per expert where the whole launch
+    //    is small - few tiles (32 experts x N = 512, 128 rows each: 63.9 us against 85.5; Mixtral down, 64 / 128
+    //    rows: 128 / 150 against 154 / 163) or under 0.5 GB of weights with a short K (Qwen3-30B down, K = 768,
+    //    64 / 128 rows: 60.5 / 89.9 against 81.1 / 105.6; DeepSeek-V2-Lite down, 96 rows: 52.3 against 87.1) -
+    //    and behind it on the large ones (DeepSeek-V3, 128 rows: 2189 against 1747)
+    if (avg > 32) {
+        // (few tiles: from 33 rows per expert where an expert is large and a second block of it costs a second
+        // read of its weights, from 65 where it is small - 32 experts x N = 512, 64 rows: 43.6 us for 64-row blocks
+        // against 63.0 - and there up to 256 rows: 74.0 against 88.5)
+        const bool large_expert = N * K >= 30000000ll;
+        if (tiles256 * 2 <= cus && avg > (large_expert ? 32 : 64) && avg <= (large_expert ? 160 : 256)) return 128;
+        if ((int64_t)num_experts * N * K <= 500000000ll && avg <= (K <= 1536 ? 224 : 112)) return 128;
+    }
+    //  * with 8 experts every block re-reads a large expert, and 64-row blocks beat blocks of the average size
+    //    (Mixtral down, 16 / 32 rows per expert: 84.2 / 86.6 us against 102.5 / 108.9)
+    if (num_experts <= 8 && avg > 8 && avg <= 40) return 64;
+    //  * the two-queue launch takes over from 12 rows per expert where an expert's N is wide, from 25 where it is
+    //    not: the row-sized ring tiles stream small experts better (Qwen3-235B gate_up, N = 3072, 16 rows: 308 us
+    //    against 373; DeepSeek-V2-Lite, 12 / 24 rows: 68.3 / 81.7 against 86.1 / 89.0)
+    if (avg > 64 || (two_queues && avg >= (N >= 4096 ? 12 : 25))) return 256;
     if (avg <= 16) return 16;
     if (avg <= 32) return 32;
     return 64;

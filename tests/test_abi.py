@@ -52,8 +52,17 @@ def test_pure_host_entry_points():
     # (256 assumed without a device), the row-sized tiles otherwise
     assert lib.mi355_grouped_block_m(8192, 256, 4096, 7168) == 256
     assert lib.mi355_grouped_block_m(2048, 256, 4096, 7168) == 16
-    assert lib.mi355_grouped_block_m(8 * 24, 8, 4096, 7168) == 32
-    assert lib.mi355_grouped_block_m(8 * 50, 8, 4096, 7168) == 64
+    assert lib.mi355_grouped_block_m(16 * 24, 16, 4096, 7168) == 32
+    assert lib.mi355_grouped_block_m(16 * 50, 16, 4096, 8192) == 64
+    assert lib.mi355_grouped_block_m(64 * 50, 64, 1024, 7168) == 128
+    # 8 experts: 64-row blocks from 9 rows per expert; few tiles or a small launch with a short K: 128-row blocks
+    assert lib.mi355_grouped_block_m(8 * 24, 8, 4096, 7168) == 64
+    assert lib.mi355_grouped_block_m(8 * 50, 8, 4096, 7168) == 128
+    assert lib.mi355_grouped_block_m(128 * 64, 128, 2048, 768) == 128
+    assert lib.mi355_grouped_block_m(128 * 300, 128, 2048, 768) == 256
+    # an expert's N under 4096: the two-queue launch from 25 rows per expert
+    assert lib.mi355_grouped_block_m(128 * 16, 128, 3072, 4096) == 16
+    assert lib.mi355_grouped_block_m(128 * 32, 128, 3072, 4096) == 256
     assert lib.mi355_block_fp8_gemm_workspace_bytes(4096, 4096, 4096, 0) == 65536  # large M: tile counters only
     assert lib.mi355_block_fp8_gemm_workspace_bytes(8, 4096, 14336, 0) > 65536
 
