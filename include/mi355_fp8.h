@@ -212,8 +212,9 @@ int mi355_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int32
  * num_pairs is only used as the row stride of expert_to_token_index / expert_to_weight (the number of (token, slot)
  * pairs in LightLLM's use); the masked expert-parallel layout passes a [E, T_pad] table with num_pairs = T_pad.
  * block_m must be one the library was built for: 16, 32, 64, 128 or 256; mi355_grouped_block_m() suggests one
- * (256 also for batches of 12 to 64 rows per expert when the launch has more tiles than compute units: that
- * suggestion counts on the workspace of mi355_grouped_workspace_bytes(), see below).
+ * from the rows per expert, the number of experts and an expert's N and K (256 also for batches of 12 to 64 rows
+ * per expert when the launch has more tiles than compute units: that suggestion counts on the workspace of
+ * mi355_grouped_workspace_bytes(), see below; 128 for small launches; 64 for models of 8 experts).
  * workspace: optional, used by block_m = 256 only: MI355_WS_COUNTER_BYTES bytes that are zero before the launch
  * (the kernel leaves them zero).  With it the launch is persistent - one workgroup per compute unit takes tiles
  * from per-XCD counters and overlaps the first requests of a tile with the stores of the previous one;
