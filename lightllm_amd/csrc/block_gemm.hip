@@ -1017,7 +1017,7 @@ extern "C" int32_t mi355_grouped_block_m(int64_t num_pairs, int32_t num_experts,
         // against 63.0 - and there up to 256 rows: 74.0 against 88.5)
         const bool large_expert = N * K >= 30000000ll;
         if (tiles256 * 2 <= cus && avg > (large_expert ? 32 : 64) && avg <= (large_expert ? 160 : 256)) return 128;
-        if ((int64_t)num_experts * N * K <= 500000000ll && avg <= (K <= 1536 ? 224 : 112)) return 128;
+        if ((int64_t)num_experts * N * K <= 500000000ll && K <= 2048 && avg <= (K <= 1536 ? 224 : 112)) return 128;
     }
     //  * with 8 experts every block re-reads a large expert, and 64-row blocks beat blocks of the average size
     //    (Mixtral down, 16 / 32 rows per expert: 84.2 / 86.6 us against 102.5 / 108.9)

@@ -54,7 +54,8 @@ def test_pure_host_entry_points():
     assert lib.mi355_grouped_block_m(2048, 256, 4096, 7168) == 16
     assert lib.mi355_grouped_block_m(16 * 24, 16, 4096, 7168) == 32
     assert lib.mi355_grouped_block_m(16 * 50, 16, 4096, 8192) == 64
-    assert lib.mi355_grouped_block_m(64 * 50, 64, 1024, 7168) == 128
+    assert lib.mi355_grouped_block_m(64 * 50, 64, 1024, 7168) == 64
+    assert lib.mi355_grouped_block_m(64 * 50, 64, 2816, 2048) == 128
     # 8 experts: 64-row blocks from 9 rows per expert; few tiles or a small launch with a short K: 128-row blocks
     assert lib.mi355_grouped_block_m(8 * 24, 8, 4096, 7168) == 64
     assert lib.mi355_grouped_block_m(8 * 50, 8, 4096, 7168) == 128
