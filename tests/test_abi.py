@@ -58,7 +58,7 @@ def test_pure_host_entry_points():
     assert lib.mi355_grouped_block_m(64 * 50, 64, 2816, 2048) == 128
     # 8 experts: 64-row blocks from 9 rows per expert; few tiles or a small launch with a short K: 128-row blocks
     assert lib.mi355_grouped_block_m(8 * 24, 8, 4096, 7168) == 64
-    assert lib.mi355_grouped_block_m(8 * 50, 8, 4096, 7168) == 128
+    assert lib.mi355_grouped_block_m(8 * 50, 8, 4096, 14336) == 128
     assert lib.mi355_grouped_block_m(128 * 64, 128, 2048, 768) == 128
     assert lib.mi355_grouped_block_m(128 * 300, 128, 2048, 768) == 256
     # an expert's N under 4096: the two-queue launch from 25 rows per expert
