@@ -441,6 +441,12 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         // streaming kernel keeps its lead, 23.8 against 27.4)
         const int64_t t64 = (N + 63) / 64;
         const Rows128Plan pl = rows128_plan(M, N, K, cus);
+        // likewise on large weights whose 64-row workgroups come to just over one per unit (N = 18432, K = 7168,
+        // 288 of them, M = 16 / 32: 27.5 / 28.4 us against 30.3 / 34.4), and under a very long K (N = 8192,
+        // K = 28672: 45.3 / 47.0 against 50.7 / 54.6; N = 7168, K = 18432: 27.2 / 28.5 against 30.9 / 31.4)
+        if (N * K >= 100000000ll && pl.tiles <= cus &&
+            ((t64 > cus && t64 * 4 <= 5 * (int64_t)cus) || K >= 18432))
+            return true;
         return t64 > 2 * (int64_t)cus && t64 <= 3 * (int64_t)cus && pl.splits == 1 && pl.tiles <= cus &&
                pl.tiles * 20 >= (int64_t)cus * 11;
     }

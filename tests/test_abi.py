@@ -193,6 +193,7 @@ def test_shape_table_choices_on_256_compute_units():
         (1, 28672, 4096): SKINNY, (8, 4096, 14336): SKINNY, (64, 4096, 14336): SKINNY, (8, 36864, 7168): SKINNY,
         (64, 128256, 4096): XSHARE, (64, 8192, 8192): SKINNY, (64, 16384, 7168): SKINNY,   # 512 / 256 workgroups
         (64, 14336, 4096): ROWS, (48, 10240, 8192): ROWS, (64, 6144, 4096): SKINNY,
+        (16, 7168, 18432): ROWS, (32, 18432, 7168): ROWS, (32, 28672, 4096): SKINNY, (8, 7168, 18432): SKINNY,
         (16, 36864, 4096): ROWS, (24, 36864, 7168): ROWS, (64, 28672, 4096): ROWS, (100, 7168, 18432): ROWS, (128, 24576, 1536): ROWS,
         (128, 2112, 7168): ROWS, (200, 4096, 14336): ROWS, (384, 4096, 14336): ROWS,
         (192, 36864, 7168): ROWS, (176, 28672, 4096): ROWS, (224, 28672, 4096): T128,   # narrower workgroups up to 208 rows

@@ -314,7 +314,7 @@ def test_rows128_column_major_scales(hip):
                                    (128, 2112, 7168), (200, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
                                    (192, 36864, 7168), (208, 24576, 1536),
                                    (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384), (48, 24576, 1536),
-                                   (64, 28672, 4096), (24, 36864, 1024), (48, 10240, 8192), (64, 14336, 4096)])
+                                   (64, 28672, 4096), (24, 36864, 1024), (48, 10240, 8192), (64, 14336, 4096), (16, 7168, 18432), (32, 18432, 7168)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
     """Model linears with 33..384 rows that the shape table gives to the weight stream with the activation block in
     LDS."""
