@@ -224,7 +224,13 @@ struct SkinnyPlan {
 static SkinnyPlan skinny_plan(int64_t M, int64_t N, int64_t K, int cus) {
     SkinnyPlan pl;
     pl.splits = 1;
-    if ((N + 63) / 64 >= cus) {
+    const int64_t t64 = (N + 63) / 64;
+    // 64-row tiles that come to just over one per unit leave half the units with twice the work of the others:
+    // narrower tiles then (N = 18432, K = 7168, 288 tiles of 64 rows, M = 1 / 16: 22.6 / 26.8 us against 27.9 /
+    // 29.9; N = 18944, K = 3584: 13.2 / 15.2 against 16.4 / 17.3); up to 1.5 per unit for M > 16, where the narrower
+    // tiles have 32 rows (N = 24576, K = 1536, M = 32 / 64: 10.3 / 15.3 against 12.2 / 18.7)
+    const bool unbalanced = t64 > cus && t64 * 4 <= (int64_t)cus * (M <= 16 ? 5 : 6);
+    if (t64 >= cus && !unbalanced) {
         // N alone gives every compute unit a workgroup: 64-row tiles, whole K
         pl.tnw = 4;
         pl.tiles = (int)((N + 63) / 64);
