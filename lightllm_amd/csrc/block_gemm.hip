@@ -490,6 +490,9 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         // flat in M (DeepSeek-V3 down, M = 208 / 240 / 256: 55.1 / 54.9 / 56.9 us against 58.4 / 60.4 / 63.3;
         // o_proj 53.1 / 52.8 / 58.1 against 54.9 / 57.5 / 57.6)
         if (M > 200 && N * K >= 100000000ll && stream_k_pays((N + 255) / 256, K / kBlockK, cus, 1)) return false;
+        // and on small weights the 128x128 tiles with K shared (N = 4096, K = 4096, M = 224 / 256: 18.9 / 19.0 us
+        // against 20.9 / 21.3; N = 7168, K = 2304, M = 256: 19.7 against 23.0)
+        if (M > 192 && N * K < 20000000ll) return false;
         if (tiles * 2 <= cus) return tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
         return tiles <= cus && (M <= 160 || (M <= kRows128NarrowMaxM && tiles * 8 >= (int64_t)cus * 7));
     }
@@ -628,6 +631,9 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
     const int64_t KB = K / kBlockK;
+    // one or two K steps: the 256x256 tile's first requests and its epilogue are most of its time (N = 7168,
+    // K = 256, M = 4096: 21.3 us for the 128x128 tiles against 27.6)
+    if (KB <= 2) return MI355_GEMM_TILE128;
     if (M > 128 && stream_k_pays(t256, KB, cus, (M + 255) / 256)) return MI355_GEMM_TILE256_STREAMK;
     // 257..384 rows leave the second 256-row tile at most half full; where the 256x256 tiles need a second round
     // anyway the 128x128 ones are ahead (N = 36864, K = 7168, M = 257 / 384: 144 / 148 us against 161 / 165) -
@@ -637,11 +643,11 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     if (t128 <= 2 * (int64_t)cus && (t256 < (int64_t)cus * 3 / 8 || KB <= 64)) {
         // a narrow N under many rows: 256x128 tiles with K shared load half as much X per product as the 128x128
         // ones and still fill the device (q_a+kv_a, N = 2112, K = 7168, M = 768 / 1024 / 1536: 35.0 / 40.6 / 50.6 us
-        // against 38.7 / 60.2 / 60.6)
+        // against 38.7 / 60.2 / 60.6; not under 12 n tiles: N = 256 / 512, M = 1024: 17.5 / 17.5 against 20.6 / 21.4)
         // ... and, from two 256-row tiles on, a wider N under a long K (N = 5120, K = 5120, M = 400 / 512: 35.4 /
         // 37.6 us against 44.7 / 45.1; N = 4096, K = 7168, M = 640: 54.6 against 60.3; on N = 1536 the 128x128 tiles
         // keep their lead, 21.8 against 25.2, and with K = 4096 too)
-        if (((M >= 768 && (N + 127) / 128 <= 24) || (M > 384 && KB >= 40 && (N + 127) / 128 >= 20)) &&
+        if (((M >= 768 && (N + 127) / 128 <= 24 && (N + 127) / 128 >= 12) || (M > 384 && KB >= 40 && (N + 127) / 128 >= 20)) &&
             tile256x128_splits(M, N, K, cus) >= 2)
             return MI355_GEMM_TILE256x128;
         return MI355_GEMM_TILE128;
