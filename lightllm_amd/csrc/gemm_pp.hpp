@@ -29,6 +29,10 @@
 //     per XCD in the caller's workspace, fetched two tiles ahead; the schedule-table row of a tile is loaded one
 //     tile ahead.  Counter words: [0..7] per-XCD, [8] workgroups that have finished; the last one to finish
 //     zeroes them again.  Without a workspace (counters == nullptr) every workgroup runs one tile.
+//     Dense launches of whole tiles (M, N multiples of 256) with an even number of K steps let the ring run on
+//     across the tile boundary: the last two steps of a tile request W and X of the first two steps of the next
+//     one, in the slots where its loop expects them, instead of repeating their own last step (M = 4096,
+//     N = 32768, K = 512, eight tiles of four steps per workgroup: 129 us against 148; N = 36864, K = 7168: 1 %).
 //   * Stream-K launch (SK, dense only): when the tiles do not fill whole rounds of the device, the K steps of all
 //     tiles - tile-major, in the dense tile order - are cut into one contiguous run per workgroup, so every compute
 //     unit does the same number of K steps.  A workgroup whose run covers only part of a tile's K range writes its
@@ -89,6 +93,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     const int KB = p.K / kBlockK, nchunk = (KB + 7) >> 3;
     const uint32_t xcd = blockIdx.x & 7u, in_xcd = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
     const bool persistent = !SK && p.counters != nullptr;
+    const bool xt_ok = !GROUPED && persistent && KB >= 2 && (KB & 1) == 0 && p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0;
     volatile uint32_t *sched = (volatile uint32_t *)(lds + (ROLES ? Cfg::roles_sched_off(KB) : Cfg::sched_off(KB)));
     // ROLES: blocks with more than 64 rows (the tile loop below) and the others (small_blocks), listed by the
     // split kernel.  The first workgroups of every XCD start on the small blocks, the others on the large ones;
@@ -321,24 +326,24 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         if (x_real[i]) dma_g2l_b128(sb + xdst[i], xk, xoff[i]);
         else dma_g2l_b32(lds0 + Cfg::kDummyOff, p.X, 0u);
     };
-    auto issue_w = [&](int stage, int kb) {
+    auto issue_w_at = [&](int stage, const uint8_t *wk) {
         const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
-        const uint8_t *wk = wg + (int64_t)kb * kBlockK;
 #pragma unroll
         for (int i = 0; i < Cfg::WI; ++i) dma_g2l_b128(sb + wdst[i], wk, woff[i]);
     };
-    auto issue_xlo = [&](int stage, int kb) {
+    auto issue_xlo_at = [&](int stage, const uint8_t *xk) {
         const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
-        const uint8_t *xk = xg + (int64_t)kb * kBlockK;
 #pragma unroll
         for (int i = 0; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
     };
-    auto issue_xhi = [&](int stage, int kb) {
+    auto issue_xhi_at = [&](int stage, const uint8_t *xk) {
         const uint32_t sb = lds0 + (uint32_t)stage * Cfg::kStage;
-        const uint8_t *xk = xg + (int64_t)kb * kBlockK;
 #pragma unroll
         for (int i = 1; i < Cfg::XI; i += 2) issue_x(i, sb, xk);
     };
+    auto issue_w = [&](int stage, int kb) { issue_w_at(stage, wg + (int64_t)kb * kBlockK); };
+    auto issue_xlo = [&](int stage, int kb) { issue_xlo_at(stage, xg + (int64_t)kb * kBlockK); };
+    auto issue_xhi = [&](int stage, int kb) { issue_xhi_at(stage, xg + (int64_t)kb * kBlockK); };
     // Scale (row, kb) sits at chunk[(kb/8) & 1][row][kb % 8].  SC4: lane l of wave w fetches steps 4*(l&1).. of row
     // 32*w + l/2.  Otherwise lane l fetches step l%8 of row l/8 of the same four 8-row groups it fetches X rows
     // for; steps past the end of K repeat the last step (never read).
@@ -425,6 +430,22 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         if (grp == 1) phase_end();
         int slot = 0;
         const int kfirst = cur.k0, klast = cur.k1 - 1;
+        // Dense persistent launches of whole tiles (M and N multiples of the tile, an even number of K steps, so that
+        // the request offsets are the same for every tile and the ring slots come out right): the last two steps
+        // of a tile, which have nothing of their own left to request, request the first two steps of the next
+        // tile instead of repeating the last step - the ring runs on across the tile boundary.
+        bool prefetch = false;
+        const uint8_t *xg_n = p.X, *wg_n = p.W;
+        if constexpr (!GROUPED && !SK) {
+            if (xt_ok) {
+                const Tile nt = make_tile(v_next, row_next);
+                prefetch = nt.valid;
+                if (prefetch) {
+                    xg_n = p.X + (int64_t)nt.m0 * p.ldx;
+                    wg_n = p.W + (int64_t)nt.n0 * p.ldw;
+                }
+            }
+        }
         for (int kb = kfirst; kb <= klast; ++kb) {
             const uint8_t *st = lds + slot * Cfg::kStage;
             const int cbuf = (kb >> 3) & 1;
@@ -455,10 +476,14 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
                 }
                 if (h == 0) {
                     if ((kb & 7) == 0 && (kb >> 3) + 1 < nchunk) issue_scales((kb >> 3) + 1);
-                    issue_xhi(slot ^ 1, min(kb + 1, klast));
+                    // (scalar selects, no branch: the body keeps its instruction order)
+                    const bool nx = prefetch && kb + 1 > klast;
+                    issue_xhi_at(slot ^ 1, (nx ? xg_n : xg) + (int64_t)(nx ? 0 : min(kb + 1, klast)) * kBlockK);
                 } else {
-                    issue_xlo(slot, min(kb + 2, klast));
-                    issue_w(slot, min(kb + 2, klast));
+                    const bool nx = prefetch && kb + 2 > klast;
+                    const int64_t ko = (int64_t)(nx ? kb + 1 - klast : min(kb + 2, klast)) * kBlockK;  // next tile: step 0 or 1
+                    issue_xlo_at(slot, (nx ? xg_n : xg) + ko);
+                    issue_w_at(slot, (nx ? wg_n : wg) + ko);
                 }
                 // everything but the last two request groups has landed: at the end of A0 that covers the second
                 // X half of this step, at the end of A1 the W rows and first X half of the next one (the scale
@@ -505,7 +530,13 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         if (cur.valid) {
             uint32_t raw[Cfg::XI + 1];
             gather(cur, raw);
-            first_requests(cur, raw);
+            if (prefetch) {  // W and X of the first two steps were requested by the last two steps above
+                setup_w(cur);
+                setup_x(cur, raw);
+                issue_scales(cur.k0 >> 3);
+            } else {
+                first_requests(cur, raw);
+            }
             // sequence number and table row for later tiles (used one and two tiles from now)
             v_next = v_after;
             row_next = load_row(v_next);

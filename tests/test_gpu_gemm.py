@@ -91,6 +91,24 @@ def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
         _check_small(xq, xs, wq, ws, c_pp)
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 8448, 512), (2048, 8448, 256), (4096, 4352, 1024), (1024, 17152, 384),
+                                   (2048, 8448 + 128, 512), (2048 - 8, 8448, 512)])
+def test_pingpong_requests_run_on_across_tiles(hip, M, N, K):
+    """Persistent launches (more tiles than compute units) of whole 256x256 tiles with an even number of K steps:
+    the last two steps of a tile request the first two of the workgroup's next tile.  Short K ranges, so that a
+    workgroup crosses several tile boundaries with two to eight steps between them; K/128 odd, a ragged N and a
+    ragged M take the plain path.  Bit-equal to the ring kernel, and against the torch fp32 dequant-matmul."""
+    print(f"gemm ping-pong across tiles M={M} N={N} K={K}", flush=True)
+    xq, xs, wq, ws = _prep(M, N, K, seed=M + N + K, device="cuda")
+    c_pp = _run(xq, xs, wq, ws, "tile256").clone()
+    assert torch.equal(c_pp.view(torch.int16), _run(xq, xs, wq, ws, "tile256").view(torch.int16))
+    c_ring = _run(xq, xs, wq, ws, "tile256ring")
+    assert torch.equal(c_pp.view(torch.int16), c_ring.view(torch.int16)), (M, N, K)
+    ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(c_pp.float(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+
+
 @pytest.mark.parametrize("K", [128, 512, 1152, 1536, 2304, 7296])
 def test_pingpong_tile_off_grid_k(hip, K):
     """K/128 not a multiple of 8 (the reference's own tuning list holds K = 512, 1152, 1536, 2304,
