@@ -29,9 +29,9 @@
 //     per XCD in the caller's workspace, fetched two tiles ahead; the schedule-table row of a tile is loaded one
 //     tile ahead.  Counter words: [0..7] per-XCD, [8] workgroups that have finished; the last one to finish
 //     zeroes them again.  Without a workspace (counters == nullptr) every workgroup runs one tile.
-//     Dense launches of whole tiles (M, N multiples of 256) with an even number of K steps let the ring run on
-//     across the tile boundary: the last two steps of a tile request W and X of the first two steps of the next
-//     one, in the slots where its loop expects them, instead of repeating their own last step (M = 4096,
+//     Dense launches with an even number of K steps let the ring run on across the boundary between two whole
+//     tiles: the last two steps of a tile request W and X of the first two steps of the next one, in the slots
+//     where its loop expects them, instead of repeating their own last step (M = 4096,
 //     N = 32768, K = 512, eight tiles of four steps per workgroup: 129 us against 148; N = 36864, K = 7168: 1 %).
 //   * Stream-K launch (SK, dense only): when the tiles do not fill whole rounds of the device, the K steps of all
 //     tiles - tile-major, in the dense tile order - are cut into one contiguous run per workgroup, so every compute
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
     const int KB = p.K / kBlockK, nchunk = (KB + 7) >> 3;
     const uint32_t xcd = blockIdx.x & 7u, in_xcd = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
     const bool persistent = !SK && p.counters != nullptr;
-    const bool xt_ok = !GROUPED && persistent && KB >= 2 && (KB & 1) == 0 && p.M % Cfg::BM == 0 && p.N % Cfg::BN == 0;
+    const bool xt_ok = !GROUPED && persistent && KB >= 2 && (KB & 1) == 0;
     volatile uint32_t *sched = (volatile uint32_t *)(lds + (ROLES ? Cfg::roles_sched_off(KB) : Cfg::sched_off(KB)));
     // ROLES: blocks with more than 64 rows (the tile loop below) and the others (small_blocks), listed by the
     // split kernel.  The first workgroups of every XCD start on the small blocks, the others on the large ones;
@@ -430,16 +430,16 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
         if (grp == 1) phase_end();
         int slot = 0;
         const int kfirst = cur.k0, klast = cur.k1 - 1;
-        // Dense persistent launches of whole tiles (M and N multiples of the tile, an even number of K steps, so that
-        // the request offsets are the same for every tile and the ring slots come out right): the last two steps
-        // of a tile, which have nothing of their own left to request, request the first two steps of the next
-        // tile instead of repeating the last step - the ring runs on across the tile boundary.
+        // Dense persistent launches with an even number of K steps (the ring slots come out right), from one whole
+        // tile to the next whole tile (the request offsets are the same): the last two steps of a tile, which have
+        // nothing of their own left to request, request the first two steps of the next tile instead of repeating
+        // the last step - the ring runs on across the tile boundary.
         bool prefetch = false;
         const uint8_t *xg_n = p.X, *wg_n = p.W;
         if constexpr (!GROUPED && !SK) {
             if (xt_ok) {
                 const Tile nt = make_tile(v_next, row_next);
-                prefetch = nt.valid;
+                prefetch = nt.valid && nt.rows == BM && nt.n0 + Cfg::BN <= p.N && cur.rows == BM && cur.n0 + Cfg::BN <= p.N;
                 if (prefetch) {
                     xg_n = p.X + (int64_t)nt.m0 * p.ldx;
                     wg_n = p.W + (int64_t)nt.n0 * p.ldw;

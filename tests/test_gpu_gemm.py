@@ -94,10 +94,11 @@ def test_pingpong_tile_equals_ring_tile(hip, M, N, K):
 @pytest.mark.parametrize("M,N,K", [(2048, 8448, 512), (2048, 8448, 256), (4096, 4352, 1024), (1024, 17152, 384),
                                    (2048, 8448 + 128, 512), (2048 - 8, 8448, 512)])
 def test_pingpong_requests_run_on_across_tiles(hip, M, N, K):
-    """Persistent launches (more tiles than compute units) of whole 256x256 tiles with an even number of K steps:
+    """Persistent launches (more tiles than compute units) of 256x256 tiles with an even number of K steps:
     the last two steps of a tile request the first two of the workgroup's next tile.  Short K ranges, so that a
-    workgroup crosses several tile boundaries with two to eight steps between them; K/128 odd, a ragged N and a
-    ragged M take the plain path.  Bit-equal to the ring kernel, and against the torch fp32 dequant-matmul."""
+    workgroup crosses several tile boundaries with two to eight steps between them; K/128 odd takes the plain path,
+    and so do the boundaries next to the partial tiles of a ragged N or M.  Bit-equal to the ring kernel, and
+    against the torch fp32 dequant-matmul."""
     print(f"gemm ping-pong across tiles M={M} N={N} K={K}", flush=True)
     xq, xs, wq, ws = _prep(M, N, K, seed=M + N + K, device="cuda")
     c_pp = _run(xq, xs, wq, ws, "tile256").clone()
