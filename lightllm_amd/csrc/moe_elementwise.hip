@@ -28,6 +28,8 @@ namespace mi355 {
 
 #pragma clang fp contract(off)
 
+// FINITE: the caller knows that g is finite (silu_mul_chunk tests a whole chunk at once).
+template <bool FINITE = false>
 __device__ __forceinline__ float silu_f32(float g) {
     const float c1 = 1.44268798828125f;                // log2(e) rounded to 16 significant bits
     const float c2ln2 = 4.888495152e-06f;              // (log2(e) - c1) * ln(2)
@@ -42,24 +44,38 @@ __device__ __forceinline__ float silu_f32(float g) {
     float y0 = g * r;
     float res = __builtin_fmaf(-y0, d, g);
     float out = __builtin_fmaf(res, r, y0);
-    // non-finite gates as g / (1 + exp(-g)) has them: NaN and -inf give NaN (-inf / inf), +inf gives +inf
-    if (__builtin_amdgcn_classf(gin, 0x007)) out = __builtin_nanf("");
-    if (__builtin_amdgcn_classf(gin, 0x200)) out = gin;
+    if constexpr (!FINITE) {
+        // non-finite gates as g / (1 + exp(-g)) has them: NaN and -inf give NaN (-inf / inf), +inf gives +inf
+        if (__builtin_amdgcn_classf(gin, 0x007)) out = __builtin_nanf("");
+        if (__builtin_amdgcn_classf(gin, 0x200)) out = gin;
+    }
     return out;
 }
 
 // bf16(silu(gate)) * up -> bf16, for the two bf16 values packed in one dword.
+template <bool FINITE = false>
 __device__ __forceinline__ uint32_t silu_mul_pk(uint32_t g2, uint32_t u2) {
     float g0 = as_f32(g2 << 16), g1 = as_f32(g2 & 0xffff0000u);
     float u0 = as_f32(u2 << 16), u1 = as_f32(u2 & 0xffff0000u);
-    uint32_t a = pack_bf16x2(silu_f32(g0), silu_f32(g1));
+    uint32_t a = pack_bf16x2(silu_f32<FINITE>(g0), silu_f32<FINITE>(g1));
     return pack_bf16x2(as_f32(a << 16) * u0, as_f32(a & 0xffff0000u) * u1);
 }
 
+// The kernels are bound by this arithmetic, so the non-finite cases (two class tests and two selects per element)
+// are tested once per chunk: a bf16 is non-finite when its exponent field is all ones, and adding 0x0080 to the
+// masked field of either half of a dword then carries into that half's top bit.
 __device__ __forceinline__ v4i silu_mul_chunk(const v4i &g, const v4i &u) {
-    v4i o;
+    uint32_t nonfinite = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = (int)silu_mul_pk((uint32_t)g[i], (uint32_t)u[i]);
+    for (int i = 0; i < 4; ++i) nonfinite |= (((uint32_t)g[i] & 0x7f807f80u) + 0x00800080u) & 0x80008000u;
+    v4i o;
+    if (nonfinite == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (int)silu_mul_pk<true>((uint32_t)g[i], (uint32_t)u[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = (int)silu_mul_pk<false>((uint32_t)g[i], (uint32_t)u[i]);
+    }
     return o;
 }
 
