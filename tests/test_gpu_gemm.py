@@ -105,6 +105,8 @@ def test_pingpong_requests_run_on_across_tiles(hip, M, N, K):
     assert torch.equal(c_pp.view(torch.int16), _run(xq, xs, wq, ws, "tile256").view(torch.int16))
     c_ring = _run(xq, xs, wq, ws, "tile256ring")
     assert torch.equal(c_pp.view(torch.int16), c_ring.view(torch.int16)), (M, N, K)
+    xs_cm = xs.t().contiguous().t()   # column-major scales: 4-byte scale requests
+    assert torch.equal(_run(xq, xs_cm, wq, ws, "tile256").view(torch.int16), c_ring.view(torch.int16)), (M, N, K)
     ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
     cos, rel = H.gemm_metrics(c_pp.float(), ref)
     assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
