@@ -118,8 +118,9 @@ static bool stream_k_pays(int64_t tiles, int64_t KB, int cus, int64_t tiles_m) {
     if (shared * 5 <= plain * 2) return true;
     // every tile shared by the same whole number of workgroups, none of which straddles two tiles, is a plain split
     // of K with half the partial tiles: it still pays at two workgroups per tile when their runs are long
-    // (N = 4096, K = 14336, M = 2048: 128 tiles, 111 us against 130; with K = 4096, 16 steps each, 51.6 against 43.7)
-    return groups % tiles == 0 && shared * 2 <= plain && shared >= 48;
+    // (N = 4096, K = 14336, M = 2048: 128 tiles, 111 us against 130; N = 16384, K = 7168, M = 512, 28 steps each: 70.0
+    // against 77.8; with K = 4096, 16 steps each, 51.6 against 43.7)
+    return groups % tiles == 0 && shared * 2 <= plain && shared >= 28;
 }
 
 static size_t stream_k_workspace(int groups) {
@@ -467,7 +468,9 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         if (M > 336 && N * K >= 100000000ll &&
             stream_k_pays(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus, (M + 255) / 256))
             return false;
-        return K / kBlockK >= 16 && N * K >= 20000000ll && tiles * 2 <= cus &&
+        // (with more than cus/4 tiles of 128 weight rows the 128x128 tiles are ahead again: N = 16384, K = 4096,
+        // M = 384: 44.7 us against 56.6; N = 12288: 43.6 against 49.1)
+        return K / kBlockK >= 16 && N * K >= 20000000ll && tiles * 4 <= cus &&
                tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
     }
     if (M > 128) {
