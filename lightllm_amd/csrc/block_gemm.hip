@@ -468,9 +468,10 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
         if (M > 336 && N * K >= 100000000ll &&
             stream_k_pays(((M + 255) / 256) * ((N + 255) / 256), K / kBlockK, cus, (M + 255) / 256))
             return false;
-        // (with more than cus/4 tiles of 128 weight rows the 128x128 tiles are ahead again: N = 16384, K = 4096,
-        // M = 384: 44.7 us against 56.6; N = 12288: 43.6 against 49.1)
-        return K / kBlockK >= 16 && N * K >= 20000000ll && tiles * 4 <= cus &&
+        // (with more than cus/4 tiles of 128 weight rows only up to 320 rows: N = 10240, K = 8192, M = 257 / 300:
+        // 49.4 / 53.4 us against 68.8 / 68.9; N = 14336, K = 5120: 48.3 / 49.7 against 54.3 / 54.0; at M = 384 the
+        // 128x128 tiles are ahead there - N = 16384, K = 4096: 44.7 against 56.6; N = 12288: 43.3 against 48.9)
+        return K / kBlockK >= 16 && N * K >= 20000000ll && tiles * 2 <= cus && (tiles * 4 <= cus || M <= 320) &&
                tiles * rows128_splits(M, N, K, cus) * 2 >= cus;
     }
     if (M > 128) {

@@ -203,7 +203,7 @@ def test_shape_table_choices_on_256_compute_units():
         (2048, 2112, 7168): STREAMK, (512, 4096, 14336): STREAMK,     # the panel split
         (240, 7168, 18432): STREAMK, (352, 7168, 18432): STREAMK, (300, 7168, 18432): ROWS,
         (768, 2112, 7168): T256x128, (512, 5120, 5120): T256x128, (1024, 2112, 7168): STREAMK, (512, 4096, 7168): STREAMK,
-        (384, 16384, 4096): T128, (512, 16384, 7168): STREAMK,
+        (384, 16384, 4096): T128, (512, 16384, 7168): STREAMK, (300, 10240, 8192): ROWS, (384, 10240, 4096): T128,
         (512, 1536, 7168): T128, (4096, 7168, 256): T128, (1024, 512, 7168): T128, (256, 4096, 4096): T128,
         (16, 256, 100): GENERIC,
     }
