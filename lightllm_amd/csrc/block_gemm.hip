@@ -515,12 +515,12 @@ static bool rows128_pays(int64_t M, int64_t N, int64_t K, int cus) {
     const SkinnyPlan sp = skinny_plan(M, N, K, cus);
     const int64_t wgs = (int64_t)sp.tiles * sp.splits;
     if (N * K >= 100000000ll) return !(sp.splits == 1 && wgs == cus);
-    // ... and on the mid-size ones (from 40 MB) where they come out as neither one nor two per unit: N = 10240,
+    // ... and on the mid-size ones (from 35 MB) where they come out as neither one nor two per unit: N = 10240,
     // K = 8192 (640 of them), M = 64: 24.5 us against 33.6; 14336 x 4096 (896): 19.6 against 24.0; 12288 x 4096 (768):
     // 18.0 against 22.4; 5120 x 13824 (640): 21.4 against 28.8.  With 512 or 256 of them it keeps its lead (8192 x
     // 8192: 21.3 against 22.9; 16384 x 4096: 18.7 against 21.3), and on smaller weights the second launch shows
     // (6144 x 4096: 12.8 against 14.6).
-    return N * K >= 40000000ll && wgs != cus && wgs != 2 * (int64_t)cus;
+    return N * K >= 35000000ll && wgs != cus && wgs != 2 * (int64_t)cus;
 }
 
 static bool rows128_limits_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t as_m, int64_t as_k, int cus) {
