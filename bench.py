@@ -290,9 +290,10 @@ def main():
         torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "decode":
-        # Llama-3-8B decode linears; the weights rotate through enough copies (> 600 MB) that no launch finds them
-        # in the 256 MB memory-side cache
-        for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down"), (128256, 4096, "lm_head")]:
+        # Llama-3-8B decode linears (and the DeepSeek-V3 dense gate_up, 264 MB); the weights rotate through enough
+        # copies (> 600 MB) that no launch finds them in the 256 MB memory-side cache
+        for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down"), (128256, 4096, "lm_head"),
+                               (36864, 7168, "deepseek-v3 gate_up")]:
             ncopies = -(-640_000_000 // (Nd * Kd))
             copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(ncopies)]
             views = [(q.t(), s.t()) for q, s in copies]
@@ -307,7 +308,8 @@ def main():
 
                 us = _time_calls(call, 2 * ncopies, ncopies)
                 gbs = gemm_bytes(Md, Nd, Kd) / us / 1e3
-                others.append({"name": f"llama3-8b {name} M={Md} N={Nd} K={Kd}", "us": round(us, 2),
+                model = "" if name.startswith("deepseek") else "llama3-8b "
+                others.append({"name": f"{model}{name} M={Md} N={Nd} K={Kd}", "us": round(us, 2),
                                "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
                                "TFLOP/s": round(2.0 * Md * Nd * Kd / us / 1e6, 2),
                                "rotated_MB": round(ncopies * Nd * Kd / 1e6)})

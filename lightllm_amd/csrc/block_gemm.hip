@@ -230,7 +230,15 @@ static SkinnyPlan skinny_plan(int64_t M, int64_t N, int64_t K, int cus) {
     // narrower tiles then (N = 18432, K = 7168, 288 tiles of 64 rows, M = 1 / 16: 22.6 / 26.8 us against 27.9 /
     // 29.9; N = 18944, K = 3584: 13.2 / 15.2 against 16.4 / 17.3); up to 1.5 per unit for M > 16, where the narrower
     // tiles have 32 rows (N = 24576, K = 1536, M = 32 / 64: 10.3 / 15.3 against 12.2 / 18.7)
-    const bool unbalanced = t64 > cus && t64 * 4 <= (int64_t)cus * (M <= 16 ? 5 : 6);
+    bool unbalanced = t64 > cus && t64 * 4 <= (int64_t)cus * (M <= 16 ? 5 : 6);
+    // up to 8 rows under a long K the 16-row tiles also win wherever the 64-row ones fill less than 84 % of their
+    // last round (N = 36864, K = 7168, 2.25 per unit, M = 1 / 8: 39.6 / 41.5 us against 45.4 / 46.2; N = 22016,
+    // K = 5120, 1.34 per unit: 19.9 / 21.4 against 22.7 / 23.4); with whole rounds they lose (N = 49152, M = 8: 41.6
+    // against 38.5), and so they do on K = 4096
+    if (M <= 8 && K >= 5120 && t64 > cus) {
+        const int64_t rounds = (t64 + cus - 1) / cus;
+        if (t64 * 25 < rounds * cus * 21) unbalanced = true;
+    }
     if (t64 >= cus && !unbalanced) {
         // N alone gives every compute unit a workgroup: 64-row tiles, whole K
         pl.tnw = 4;
