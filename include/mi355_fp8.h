@@ -95,8 +95,9 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
  * block_n = block_k = 128 for the tiled kernels; any other positive block sizes run on the plain kernel
  * (MI355_GEMM_AUTO or MI355_GEMM_GENERIC), the last K block may be partial.
  *
- * `variant` picks the kernel: MI355_GEMM_AUTO applies the built-in shape table (and falls back to
- * MI355_GEMM_TILE128 when a limit of the streaming kernel - 32-bit row offsets, workspace - is not met); the
+ * `variant` picks the kernel: MI355_GEMM_AUTO applies the built-in shape table (and falls back, kernel by kernel,
+ * to one that runs when a limit of the chosen kernel - 32-bit row offsets, LDS, workspace - is not met: it never
+ * fails for want of a workspace, see mi355_block_fp8_gemm_plan); the
  * others force one (for tests and tuning) and report such a limit as an error.  Split-K variants need `ws` of at least
  * mi355_block_fp8_gemm_workspace_bytes() bytes, whose first MI355_WS_COUNTER_BYTES must be zero
  * on the first call; the kernels leave them zero again, so one zero-initialised buffer serves every call
@@ -127,6 +128,13 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
  * the codes above; MI355_GEMM_GENERIC when K is not a multiple of 128).  No counterpart in the reference, whose
  * autotuner picks tile sizes at run time (fp8w8a8_block_gemm_kernel.py:120-146); for logs and tests. */
 int32_t mi355_block_fp8_gemm_variant(int64_t M, int64_t N, int64_t K);
+
+/* The kernel an MI355_GEMM_AUTO call launches (first) for a packed, 16-byte aligned problem when it is handed a
+ * workspace of `ws_bytes` bytes (0 = none), on a device with `cus` compute units (<= 0: the current device): the
+ * table's choice, or the kernel it falls back to where that choice's workspace is missing - the chain always ends in
+ * a kernel that runs without one, so AUTO never returns MI355_EWORKSPACE.  Launches nothing.  No counterpart in the
+ * reference; for tests of the table off the device it was measured on, and for callers that size workspaces. */
+int32_t mi355_block_fp8_gemm_plan(int64_t M, int64_t N, int64_t K, size_t ws_bytes, int32_t cus);
 
 /* Bytes of workspace the launch plan of the CURRENT device needs for this shape and variant (0 = none). */
 size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant);
@@ -240,6 +248,19 @@ int mi355_grouped_block_fp8_gemm_dtype(const void *Xq, const float *Xs, const vo
                                        int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
                                        int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
                                        void *ws, size_t ws_bytes, int32_t out_dtype, void *stream);
+
+/* The same with a per-expert bias (ADD_BIAS, grouped_fused_moe.py:501-503, 702-707): bias [E, N] of `bias_dtype`
+ * (MI355_DTYPE_BF16 / _F16 / _F32), expert stride bias_stride_e elements, widened to fp32 and added to the
+ * accumulator before the routed weight is applied (:709-715):
+ *     out[idx, :] = cast( (blockscaled(Xq[row,:] . W[e]^T) + bias[e, :]) * (mul_routed_weight ? weight : 1) ).
+ * bias == NULL is mi355_grouped_block_fp8_gemm_dtype. */
+int mi355_grouped_block_fp8_gemm_bias(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                      const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                      const int32_t *expert_token_num, const int32_t *table, int64_t table_rows,
+                                      int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
+                                      int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
+                                      void *ws, size_t ws_bytes, int32_t out_dtype, const void *bias,
+                                      int32_t bias_dtype, int64_t bias_stride_e, void *stream);
 
 /* ---- element-wise steps between / after the two expert GEMMs ------------------------------------------------ */
 

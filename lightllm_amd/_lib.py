@@ -24,6 +24,7 @@ SIGNATURES = {
     "mi355_group_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _f32, _i64, _i64, _vp]),
     "mi355_block_weight_quant_fp8": (_c.c_int, [_vp, _i32, _vp, _vp, _i64, _i64, _i32, _vp]),
     "mi355_block_fp8_gemm_variant": (_i32, [_i64, _i64, _i64]),
+    "mi355_block_fp8_gemm_plan": (_i32, [_i64, _i64, _i64, _sz, _i32]),
     "mi355_block_fp8_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "mi355_block_fp8_gemm_noalloc": (
         _c.c_int,
@@ -57,6 +58,11 @@ SIGNATURES = {
         _c.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp,
          _c.c_size_t, _i32, _vp],
+    ),
+    "mi355_grouped_block_fp8_gemm_bias": (
+        _c.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i64, _i32, _i32, _i64, _i64, _i32, _vp, _vp,
+         _c.c_size_t, _i32, _vp, _i32, _i64, _vp],
     ),
     "mi355_silu_and_mul": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "mi355_silu_and_mul_ex": (_c.c_int, [_vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _f32, _f32, _vp]),
@@ -123,32 +129,46 @@ def require_cuda(*tensors: torch.Tensor) -> None:
             raise Mi355Error("lightllm_amd operators run on the GPU only; got a CPU tensor")
 
 
-_workspaces = {}
+_workspaces = {}  # (device index, stream handle or _GRAPH) -> buffer
 _retired = []  # outgrown workspaces: kept alive, a captured HIP graph may still hold their address
 
 
-def workspace(device: torch.device, nbytes: int, stream: int = None) -> torch.Tensor:
-    """Per (device, stream) scratch for split-K and persistent launches: zero-initialised once, grown on demand.
+_GRAPH = "graph"  # key of a device's workspace for launches recorded into HIP graphs
 
-    The kernels leave the counter words zero, so the buffer is never cleared again.  A buffer that has been
-    handed out is never freed: when a later call needs more, a larger one takes its place for new launches and
-    the old one stays allocated, because a HIP graph captured earlier has its address baked in and keeps
-    using it on replay.  Growing allocates, so callers that capture graphs run each shape once before capturing
-    (as with any use of the torch allocator).
+
+def workspace(device: torch.device, nbytes: int, stream: int = None) -> torch.Tensor:
+    """Scratch for split-K and persistent launches: zero-initialised once, grown on demand.
+
+    Eager launches use one buffer per (device, stream).  Launches recorded under HIP graph capture use one buffer
+    per device that every eager call sizes along with its own: the capture stream is not the stream of the warm-up
+    run (``torch.cuda.graph`` captures on a side stream), so a buffer looked up by stream would be missed there and
+    allocated - and zero-filled on every replay - inside the graph.  After the shape has run once outside a
+    capture, capturing it allocates nothing.  A capture of a shape that never ran eagerly still works: it gets a
+    buffer from the graph's own pool, zero-filled by a node of the graph.
+
+    The kernels leave the counter words zero, so a buffer is never cleared again.  A buffer that has been handed
+    out is never freed: when a later call needs more, a larger one takes its place for new launches and the old
+    one stays allocated, because a graph captured earlier has its address baked in and keeps using it on replay.
+    Graphs of one device share that device's buffer: replay them one at a time (launches that overlap in time on
+    one workspace race).
     """
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           stream_ptr(device) if stream is None else stream)
+    dev = device.index if device.index is not None else torch.cuda.current_device()
+    capturing = torch.cuda.is_current_stream_capturing()
+    key = (dev, _GRAPH) if capturing else (dev, stream_ptr(device) if stream is None else stream)
     buf = _workspaces.get(key)
     if buf is not None and buf.numel() >= nbytes:
         return buf
+    if capturing:
+        return torch.zeros(max(nbytes, WS_COUNTER_BYTES), dtype=torch.uint8, device=device)
+    size = max(nbytes, WS_COUNTER_BYTES + (32 << 20))
     with _lock:
-        buf = _workspaces.get(key)
-        if buf is None or buf.numel() < nbytes:
-            if buf is not None:
-                _retired.append(buf)
-            size = max(nbytes, WS_COUNTER_BYTES + (32 << 20))
-            buf = torch.zeros(size, dtype=torch.uint8, device=device)
-            _workspaces[key] = buf
+        for k in (key, (dev, _GRAPH)):
+            old = _workspaces.get(k)
+            if old is None or old.numel() < nbytes:
+                if old is not None:
+                    _retired.append(old)
+                _workspaces[k] = torch.zeros(size, dtype=torch.uint8, device=device)
+        buf = _workspaces[key]
     return buf
 
 

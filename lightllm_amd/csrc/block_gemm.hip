@@ -274,13 +274,13 @@ static size_t skinny_workspace(int64_t M, const SkinnyPlan &pl) {
 
 // Preconditions of the stream kernel beyond the fast layout.
 static int skinny_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t as_m, int cus,
-                        const void *ws, size_t ws_bytes) {
+                        bool ws_usable, size_t ws_bytes) {
     if (M > 64) return MI355_EUNSUPPORTED;
     // rows are addressed from the matrix bases with 32-bit byte offsets
     if (N * ldw >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)) return MI355_EUNSUPPORTED;
     const SkinnyPlan pl = skinny_plan(M, N, K, cus);
     if ((int64_t)pl.tiles * 4 > MI355_WS_COUNTER_BYTES) return MI355_EUNSUPPORTED;
-    if (pl.splits > 1 && (!ws || ws_bytes < skinny_workspace(M, pl) || ((uintptr_t)ws & 15))) return MI355_EWORKSPACE;
+    if (pl.splits > 1 && (!ws_usable || ws_bytes < skinny_workspace(M, pl))) return MI355_EWORKSPACE;
     return MI355_OK;
 }
 
@@ -700,20 +700,15 @@ static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus) {
     return n1 > 0 && n1 < N ? n1 : 0;
 }
 
-}  // namespace mi355
-
-using namespace mi355;
-
-extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant) {
+// Workspace of a launch plan on a device with `cus` compute units.
+static size_t workspace_bytes_for(int64_t M, int64_t N, int64_t K, int32_t variant, int cus) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % kBlockK != 0) return 0;
-    // sized from the launch plan of the current device (256 compute units when no device is visible)
-    const int cus = device_cus();
     if (variant == MI355_GEMM_AUTO) {
         variant = pick_variant(M, N, K, cus);
         const int64_t n1 = variant == MI355_GEMM_TILE256 ? n_split_rows(M, N, K, cus) : 0;
         if (n1 > 0) {
-            const size_t rest = mi355_block_fp8_gemm_workspace_bytes(M, N - n1, K, MI355_GEMM_AUTO);
+            const size_t rest = workspace_bytes_for(M, N - n1, K, MI355_GEMM_AUTO, cus);
             return rest > (size_t)MI355_WS_COUNTER_BYTES ? rest : (size_t)MI355_WS_COUNTER_BYTES;
         }
     }
@@ -741,6 +736,47 @@ extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int
     if (variant != MI355_GEMM_SKINNY || M > 64) return 0;
     const SkinnyPlan pl = skinny_plan(M, N, K, cus);
     return pl.splits > 1 ? skinny_workspace(M, pl) : 0;
+}
+
+// The kernel an AUTO call launches (first) for a problem in the fast layout: the table's choice, or - where a limit
+// of that kernel is not met or its workspace is missing - the next kernel with fewer preconditions.  The chain ends
+// in tiles that take every fast layout and run unsplit without a workspace, so AUTO never fails for want of one.
+// The 256-row stream is checked first because the table's other choice for its shapes can be any of the kernels
+// checked after it.
+static int resolve_auto(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t as_m, int64_t as_k,
+                        bool ws_usable, size_t ws_bytes, int cus) {
+    int variant = pick_variant(M, N, K, cus);
+    if (variant == MI355_GEMM_ROWS128 &&
+        (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus) ||
+         (rows128_splits(M, N, K, cus) > 1 && (!ws_usable || ws_bytes < rows128_workspace(M, N, K, cus)))))
+        variant = pick_variant(M, N, K, cus, false);
+    // stream-K needs its partial-tile slots; without them the plain tile loop gives the same result
+    if (variant == MI355_GEMM_TILE256_STREAMK &&
+        (!ws_usable || ws_bytes < workspace_bytes_for(M, N, K, variant, cus)))
+        variant = MI355_GEMM_TILE256;
+    if (variant == MI355_GEMM_SKINNY_XSHARE &&
+        (N * ldw >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32) ||
+         (N + XshareCfg::BN - 1) / XshareCfg::BN * 4 > MI355_WS_COUNTER_BYTES))
+        variant = MI355_GEMM_TILE128;
+    if (variant == MI355_GEMM_SKINNY &&
+        skinny_check(M, N, K, lda, ldw, as_m, cus, ws_usable, ws_bytes) != MI355_OK)
+        variant = MI355_GEMM_TILE128;
+    return variant;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" size_t mi355_block_fp8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int32_t variant) {
+    // sized from the launch plan of the current device (256 compute units when no device is visible)
+    return workspace_bytes_for(M, N, K, variant, device_cus());
+}
+
+extern "C" int32_t mi355_block_fp8_gemm_plan(int64_t M, int64_t N, int64_t K, size_t ws_bytes, int32_t cus) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % kBlockK != 0) return MI355_GEMM_GENERIC;
+    if (cus <= 0) cus = device_cus();
+    return resolve_auto(M, N, K, K, K, K / kBlockK, 1, ws_bytes > 0, ws_bytes, cus);
 }
 
 /* The kernel the shape table picks for a packed, aligned problem on the current device (256 compute units when no
@@ -777,24 +813,9 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
                       as_m >= 0 && as_k >= 0;
     const bool was_auto = variant == MI355_GEMM_AUTO;
     if (was_auto) {
-        variant = fast && blocks128 ? pick_variant(M, N, K, cus) : MI355_GEMM_GENERIC;
-        // stream-K needs its partial-tile slots; without them the plain tile loop gives the same result
-        if (variant == MI355_GEMM_TILE256_STREAMK &&
-            (!ws || ws_bytes < mi355_block_fp8_gemm_workspace_bytes(M, N, K, variant) || ((uintptr_t)ws & 15)))
-            variant = MI355_GEMM_TILE256;
-        // the stream kernel's own limits are not errors under AUTO: the 128x128 tile takes every fast layout
-        // and runs unsplit without a workspace
-        if (variant == MI355_GEMM_SKINNY_XSHARE &&
-            (N * ldb_n >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)))
-            variant = MI355_GEMM_TILE128;
-        // the table's other choice where a limit of the 256-row stream is not met or its partial sums have no room
-        if (variant == MI355_GEMM_ROWS128 &&
-            (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus) ||
-             (rows128_splits(M, N, K, cus) > 1 &&
-              (!ws || ws_bytes < rows128_workspace(M, N, K, cus) || ((uintptr_t)ws & 15)))))
-            variant = pick_variant(M, N, K, cus, false);
-        if (variant == MI355_GEMM_SKINNY && skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes) != MI355_OK)
-            variant = MI355_GEMM_TILE128;
+        const bool ws_usable = ws && ((uintptr_t)ws & 15) == 0;
+        variant = fast && blocks128 ? resolve_auto(M, N, K, lda, ldb_n, as_m, as_k, ws_usable, ws_bytes, cus)
+                                    : MI355_GEMM_GENERIC;
     }
     if (was_auto && variant == MI355_GEMM_TILE256) {
         const int64_t n1 = n_split_rows(M, N, K, cus);
@@ -926,7 +947,7 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
             }
         }
         case MI355_GEMM_SKINNY: {
-            const int ok = skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws, ws_bytes);
+            const int ok = skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws && ((uintptr_t)ws & 15) == 0, ws_bytes);
             if (ok != MI355_OK) return ok;
             const SkinnyPlan pl = skinny_plan(M, N, K, cus);
             switch (skinny_mt(M)) {
@@ -1070,8 +1091,12 @@ static int grouped_block_fp8_gemm_impl(const void *Xq, const float *Xs, const vo
                                        const int32_t *expert_token_num, const int32_t *table, int64_t table_rows,
                                        int32_t block_m, int64_t num_pairs, int64_t num_tokens, int32_t num_experts,
                                        int32_t topk_num, int64_t N, int64_t K, int32_t mul_routed_weight, void *out,
-                                       void *ws, size_t ws_bytes, int32_t out_dtype, void *stream) {
+                                       void *ws, size_t ws_bytes, int32_t out_dtype, const void *bias,
+                                       int32_t bias_dtype, int64_t bias_stride_e, void *stream) {
     if (out_dtype != MI355_DTYPE_BF16 && out_dtype != MI355_DTYPE_F16) return MI355_EUNSUPPORTED;
+    if (bias && bias_dtype != MI355_DTYPE_BF16 && bias_dtype != MI355_DTYPE_F16 && bias_dtype != MI355_DTYPE_F32)
+        return MI355_EUNSUPPORTED;
+    if (bias && bias_stride_e < 0) return MI355_EINVAL;
     if (num_pairs < 0 || num_tokens < 0 || num_experts <= 0 || topk_num <= 0 || N < 0 || K < 0 || table_rows < 0)
         return MI355_EINVAL;
     if (num_pairs == 0 || N == 0 || table_rows == 0) return MI355_OK;
@@ -1112,6 +1137,9 @@ static int grouped_block_fp8_gemm_impl(const void *Xq, const float *Xs, const vo
     a.num_pairs = (int)num_pairs;
     a.topk = topk_num;
     a.mul_weight = mul_routed_weight ? 1 : 0;
+    a.bias = bias;
+    a.bias_e = bias_stride_e;
+    a.bias_dtype = bias_dtype;
     a.tiles_m = (int)table_rows;
 
     auto finish = [&](int BN) {
@@ -1142,7 +1170,7 @@ extern "C" int mi355_grouped_block_fp8_gemm(const void *Xq, const float *Xs, con
                                             size_t ws_bytes, void *stream) {
     return grouped_block_fp8_gemm_impl(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weight, expert_token_num, table,
                                        table_rows, block_m, num_pairs, num_tokens, num_experts, topk_num, N, K,
-                                       mul_routed_weight, out, ws, ws_bytes, MI355_DTYPE_BF16, stream);
+                                       mul_routed_weight, out, ws, ws_bytes, MI355_DTYPE_BF16, nullptr, 0, 0, stream);
 }
 
 extern "C" int mi355_grouped_block_fp8_gemm_dtype(const void *Xq, const float *Xs, const void *W, const float *Ws,
@@ -1155,5 +1183,19 @@ extern "C" int mi355_grouped_block_fp8_gemm_dtype(const void *Xq, const float *X
                                                   void *stream) {
     return grouped_block_fp8_gemm_impl(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weight, expert_token_num, table,
                                        table_rows, block_m, num_pairs, num_tokens, num_experts, topk_num, N, K,
-                                       mul_routed_weight, out, ws, ws_bytes, out_dtype, stream);
+                                       mul_routed_weight, out, ws, ws_bytes, out_dtype, nullptr, 0, 0, stream);
+}
+
+extern "C" int mi355_grouped_block_fp8_gemm_bias(const void *Xq, const float *Xs, const void *W, const float *Ws,
+                                                 const int32_t *expert_to_token_index, const float *expert_to_weight,
+                                                 const int32_t *expert_token_num, const int32_t *table,
+                                                 int64_t table_rows, int32_t block_m, int64_t num_pairs,
+                                                 int64_t num_tokens, int32_t num_experts, int32_t topk_num, int64_t N,
+                                                 int64_t K, int32_t mul_routed_weight, void *out, void *ws,
+                                                 size_t ws_bytes, int32_t out_dtype, const void *bias,
+                                                 int32_t bias_dtype, int64_t bias_stride_e, void *stream) {
+    return grouped_block_fp8_gemm_impl(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weight, expert_token_num, table,
+                                       table_rows, block_m, num_pairs, num_tokens, num_experts, topk_num, N, K,
+                                       mul_routed_weight, out, ws, ws_bytes, out_dtype, bias, bias_dtype,
+                                       bias_stride_e, stream);
 }

@@ -568,6 +568,9 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
             const int nbase = done.n0 + wave_n * WNS;
             const int32_t *idx_list = GROUPED ? p.e2t_index + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
             const float *w_list = GROUPED ? p.e2t_weight + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
+            const bool add_bias = GROUPED && p.bias != nullptr;
+            float bias[4 * TN];
+            if (add_bias) lane_bias<TN>(p, done.expert, nbase, g4, bias);
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int rl = wave_m * WMS + 16 * i + r16;
@@ -585,7 +588,9 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = GROUPED ? acc[i][j][vv] * rw : acc[i][j][vv];
+                    for (int vv = 0; vv < 4; ++vv)
+                        o[4 * j + vv] =
+                            GROUPED ? (add_bias ? acc[i][j][vv] + bias[4 * j + vv] : acc[i][j][vv]) * rw : acc[i][j][vv];
                 if (p.vec_store && nbase + WNS <= p.N) {
 #pragma unroll
                     for (int h = 0; h < TN / 2; ++h)

@@ -160,6 +160,9 @@ __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *l
     // n0 + 64*wave + lane_col(g4, 2h) + [0, 8)
     const int nbase = n0 + wave * WNS;
     const float *w_list = p.e2t_weight + (int64_t)expert * p.num_pairs + m0;
+    const bool add_bias = p.bias != nullptr;
+    float bias[4 * TN];
+    if (add_bias) lane_bias<TN>(p, expert, nbase, g4, bias);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int rl = 16 * i + r16;
@@ -171,7 +174,8 @@ __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *l
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int vv = 0; vv < 4; ++vv) o[4 * j + vv] = acc[i][j][vv] * rw;
+            for (int vv = 0; vv < 4; ++vv)
+                o[4 * j + vv] = (add_bias ? acc[i][j][vv] + bias[4 * j + vv] : acc[i][j][vv]) * rw;
         if (p.vec_store && nbase + WNS <= p.N) {
 #pragma unroll
             for (int h = 0; h < TN / 2; ++h)

@@ -64,6 +64,9 @@ struct GemmArgs {
     const int32_t *e_num;        // [E]
     int64_t w_e, ws_e;           // expert strides of W (bytes) and Ws (elements)
     int32_t num_pairs, topk, mul_weight;
+    const void *bias;            // [E,N] added to the fp32 accumulator before the routed weight, or nullptr
+    int64_t bias_e;              // its expert stride (elements)
+    int32_t bias_dtype;          // MI355_DTYPE_*
     // grouped launch with two kinds of workgroups (gemm_pp.hpp): row indices of the schedule table split by size
     const int32_t *lists;        // [0] = blocks with more than 64 rows, [1] = the others, then the two index lists
     int32_t small_first;         // workgroups per XCD that start on the small blocks
@@ -79,6 +82,23 @@ struct GemmArgs {
 template <int TN>
 __device__ __forceinline__ constexpr int lane_col(int g, int tn) {
     return TN == 1 ? 4 * g : 32 * (tn >> 1) + 8 * g + 4 * (tn & 1);
+}
+
+// The per-expert bias of the grouped launches: the values of the 4*TN output columns a lane holds (the same for
+// every row of the tile), widened to fp32.  Columns past N repeat the last one (never stored).
+__device__ __forceinline__ float bias_value(const void *bias, int dtype, int64_t i) {
+    if (dtype == MI355_DTYPE_F32) return ((const float *)bias)[i];
+    const uint16_t h = ((const uint16_t *)bias)[i];
+    if (dtype == MI355_DTYPE_F16) return (float)__builtin_bit_cast(_Float16, h);
+    return as_f32((uint32_t)h << 16);
+}
+template <int TN>
+__device__ __forceinline__ void lane_bias(const GemmArgs &p, int expert, int nbase, int g4, float (&b)[4 * TN]) {
+#pragma unroll
+    for (int e = 0; e < 4 * TN; ++e) {
+        const int c = min(nbase + lane_col<TN>(g4, e >> 2) + (e & 3), p.N - 1);
+        b[e] = bias_value(p.bias, p.bias_dtype, (int64_t)expert * p.bias_e + c);
+    }
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE>
@@ -166,8 +186,9 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     const uint8_t *Wbase = p.W;
     const float *Wsbase = p.Ws;
     int rows_valid;  // number of valid rows in this tile
+    int expert = 0;
     if constexpr (GROUPED) {
-        const int expert = p.table[tile_m * 4 + 0];
+        expert = p.table[tile_m * 4 + 0];
         if (expert < 0) return;
         const int mi = p.table[tile_m * 4 + 1];
         const int cnt = p.e_num[expert];
@@ -384,6 +405,9 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     // ---- epilogue: lane (r16, g4) holds, for each tm, row m = wave_m*WMS + 16*tm + r16 and, for each MFMA block
     // tn, the 4 columns n0 + wave_n*WNS + lane_col(g4, tn) + [0, 4).
     const int nbase = n0 + wave_n * WNS;
+    const bool add_bias = GROUPED && p.bias != nullptr;
+    float bias[4 * TN];
+    if (add_bias) lane_bias<TN>(p, expert, nbase, g4, bias);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int rl = wave_m * WMS + 16 * i + r16;
@@ -401,7 +425,8 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) o[4 * j + v] = GROUPED ? acc[i][j][v] * rw : acc[i][j][v];
+            for (int v = 0; v < 4; ++v)
+                o[4 * j + v] = GROUPED ? (add_bias ? acc[i][j][v] + bias[4 * j + v] : acc[i][j][v]) * rw : acc[i][j][v];
         if (p.vec_store && nbase + WNS <= p.N) {
             if constexpr (TN == 1) {
                 *(v2i *)(cp + lane_col<TN>(g4, 0)) = v2i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16)};

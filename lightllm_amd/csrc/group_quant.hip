@@ -21,7 +21,7 @@ template <int UNROLL, bool ROW_MAJOR_SCALES>
 __global__ __launch_bounds__(256) void group_quant_kernel(const v4i *__restrict__ x, v2i *__restrict__ q,
                                                           float *__restrict__ s, uint32_t total_chunks,
                                                           uint32_t groups_per_row, int64_t s_stride_m,
-                                                          int64_t s_stride_g, float eps, int eps_is_default) {
+                                                          int64_t s_stride_g) {
     const uint32_t base = blockIdx.x * (256u * UNROLL) + threadIdx.x;
     v4i v[UNROLL];
 #pragma unroll
@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const v4i *__restrict_
         if (c < total_chunks) {  // total_chunks is a multiple of 16: a DPP row is active or idle as a whole
             v2i o;
             float sc;
-            quant_chunk(v[u], eps, eps_is_default != 0, o, sc);
+            quant_chunk(v[u], o, sc);
             __builtin_nontemporal_store(o, q + c);
             if ((threadIdx.x & 15u) == 0) {
                 uint32_t g = c >> 4;
@@ -67,6 +67,14 @@ __global__ __launch_bounds__(256) void group_quant_wide_kernel(const T *__restri
         for (int i = 0; i < 4; ++i) {
             f[i] = as_f32((uint32_t)a[i]);
             f[4 + i] = as_f32((uint32_t)b[i]);
+        }
+    } else if constexpr (sizeof(T) == 2 && !__is_same(T, _Float16)) {
+        // bf16 bits (T = uint16_t): the path of a non-default eps, whose floor is no bf16 value
+        const v4i a = __builtin_nontemporal_load((const v4i *)x + c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = as_f32((uint32_t)a[i] << 16);
+            f[2 * i + 1] = as_f32((uint32_t)a[i] & 0xffff0000u);
         }
     } else {
         typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -222,10 +230,16 @@ extern "C" int mi355_group_quant_fp8(const void *x, int32_t x_dtype, void *q, fl
     if (x_dtype == MI355_DTYPE_F16)
         return launch(group_quant_wide_kernel<_Float16>, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
                       (const _Float16 *)x, (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps);
+    // The two-FMA quotient of the bf16 kernel is proven for scales RN(amax/448) of a bf16 amax and of the default
+    // floor 1e-10 only; with any other eps a group below the floor has a scale outside that set, so such calls take
+    // the kernel with true divisions (fp8act_quant_kernel.py:63-113 hands eps through to the kernel).
+    if (!eps_default)
+        return launch(group_quant_wide_kernel<uint16_t>, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st,
+                      (const uint16_t *)x, (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps);
     if (row_major)
         return launch((group_quant_kernel<UNROLL, true>), dim3(blocks), dim3(256), 0, st, (const v4i *)x,
-                           (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps, eps_default);
+                           (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g);
     else
         return launch((group_quant_kernel<UNROLL, false>), dim3(blocks), dim3(256), 0, st, (const v4i *)x,
-                           (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g, eps, eps_default);
+                           (v2i *)q, s, (uint32_t)chunks, G, s_stride_m, s_stride_g);
 }

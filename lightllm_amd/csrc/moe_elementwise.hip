@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void silu_mul_quant_kernel(const uint16_t *__r
             v4i a = silu_mul_chunk(g[k], u[k]);
             v2i o;
             float sc;
-            quant_chunk(a, 1e-10f, true, o, sc);
+            quant_chunk(a, o, sc);
             __builtin_nontemporal_store(o, q + (base + k * 256u));
             if ((threadIdx.x & 15u) == 0)
                 s[(int64_t)p[k].row * s_stride_m + (int64_t)(p[k].col >> 4) * s_stride_g] = sc;

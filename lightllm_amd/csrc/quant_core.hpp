@@ -7,7 +7,7 @@
 // Doing two IEEE divisions per element would make the kernels VALU-bound, so:
 //   * s = amax/448 is formed as q0 = amax*c, s = fma(fma(-q0,448,amax), c, q0) with c = RN(1/448);
 //     this equals RN(amax/448) for every bf16 amax and for the default eps (checked exhaustively on
-//     the CPU); for any other eps a true division is taken.
+//     the CPU); calls with any other eps do not come here (they take quant_chunk_f32).
 //   * x/s is formed as y0 = x*r, y = fma(fma(-y0,s,x), r, y0) with r = RN(1/s) (a true division,
 //     once per lane).  For every pair (bf16 amax, bf16 |x| <= amax) this equals RN(x/s) whenever
 //     |x/s| >= 2^-10, and below that both round to the e4m3 zero - also checked exhaustively on the CPU
@@ -94,8 +94,9 @@ __device__ __forceinline__ void quant_chunk_f32(const float (&f)[8], float eps, 
     scale = s;
 }
 
-// Quantize one 16-byte chunk of bf16; the group amax is shared through the DPP row.
-__device__ __forceinline__ void quant_chunk(const v4i &v, float eps, bool eps_is_default, v2i &out, float &scale) {
+// Quantize one 16-byte chunk of bf16 with the default floor eps = 1e-10; the group amax is shared through the DPP row.
+__device__ __forceinline__ void quant_chunk(const v4i &v, v2i &out, float &scale) {
+    constexpr float eps = 1e-10f;
     uint32_t d0 = (uint32_t)v[0], d1 = (uint32_t)v[1], d2 = (uint32_t)v[2], d3 = (uint32_t)v[3];
     // |x| as integers: for non-negative floats the integer order is the float order.
     uint32_t m = pk_max_u16(pk_max_u16(d0 & 0x7fff7fffu, d1 & 0x7fff7fffu),
@@ -110,14 +111,9 @@ __device__ __forceinline__ void quant_chunk(const v4i &v, float eps, bool eps_is
     }
     float amax = as_f32(mx);
     amax = amax > eps ? amax : eps;
-    float s;
-    if (eps_is_default) {
-        const float c = 1.0f / 448.0f;
-        float q0 = amax * c;
-        s = __builtin_fmaf(__builtin_fmaf(-q0, 448.0f, amax), c, q0);
-    } else {
-        s = amax / 448.0f;
-    }
+    const float c = 1.0f / 448.0f;
+    float q0 = amax * c;
+    const float s = __builtin_fmaf(__builtin_fmaf(-q0, 448.0f, amax), c, q0);
     float r = 1.0f / s;
     float f[8];
     f[0] = as_f32(d0 << 16); f[1] = as_f32(d0 & 0xffff0000u);

@@ -1,10 +1,13 @@
 from .grouped_fused_moe import (  # noqa: F401
+    fused_experts,
     fused_experts_impl,
     grouped_matmul,
+    inplace_fused_experts_impl,
     moe_align,
     moe_align1,
     moe_align2,
     moe_align_fused,
+    outplace_fused_experts_impl,
 )
 from .moe_silu_and_mul import silu_and_mul_fwd  # noqa: F401
 from .moe_silu_and_mul_mix_quant_ep import (  # noqa: F401

@@ -123,10 +123,10 @@ def grouped_matmul(
 
     token_inputs bf16 [T,K] (quantized here per 1x128 group, reference :862-875) or, as an extension,
     already-quantized e4m3fn with ``token_input_scale`` [T,K/128]; expert_weights e4m3fn [E,N,K];
-    expert_to_weights_scale fp32 [E,N/128,K/128]; out bf16 [T*topk, N].
+    expert_to_weights_scale fp32 [E,N/128,K/128]; out bf16 [T*topk, N]; ``bias`` [E, N] (bf16, fp16 or fp32) is
+    added to the fp32 accumulator before the routed weight (reference :702-715).
     """
     assert use_fp8_w8a8, "only the fp8 block-quantized branch is implemented on gfx950"
-    assert bias is None, "per-expert bias is not supported by the fp8 block branch"
     expert_num, n, k = expert_weights.shape
     assert token_inputs.shape[1] == k
     assert expert_to_token_index.shape == expert_to_weights.shape
@@ -143,7 +143,9 @@ def grouped_matmul(
         "weights must be 128x128 block-quantized"
     )
     assert out.dtype in (torch.bfloat16, torch.float16) and out.shape[1] == n
-    _lib.require_cuda(token_inputs, expert_weights, out)
+    if bias is not None:
+        assert bias.shape == (expert_num, n) and bias.stride(1) == 1 and bias.dtype in _lib.DTYPE_CODES
+    _lib.require_cuda(token_inputs, expert_weights, out, bias)
     lib = _lib.lib()
 
     if token_inputs.dtype == torch.float8_e4m3fn:
@@ -167,13 +169,14 @@ def grouped_matmul(
     # the 256-row launch is persistent when it gets the (zero at rest) tile counters of this stream's workspace
     # (and, given room for the two block lists, runs the blocks of few rows on the weight-streaming tile)
     ws = _lib.workspace(out.device, lib.mi355_grouped_workspace_bytes(table.shape[0])) if block_m == 256 else None
-    code = lib.mi355_grouped_block_fp8_gemm_dtype(
+    code = lib.mi355_grouped_block_fp8_gemm_bias(
         token_inputs.data_ptr(), token_input_scale.data_ptr(), expert_weights.data_ptr(),
         expert_to_weights_scale.data_ptr(), expert_to_token_index.data_ptr(), expert_to_weights.data_ptr(),
         expert_to_token_num.data_ptr(), table.data_ptr(), table.shape[0], block_m, token_num_mul_topk_num,
         token_inputs.shape[0], expert_num, topk_num, n, k, 1 if mul_routed_weight else 0, out.data_ptr(),
         ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _lib.DTYPE_CODES[out.dtype],
-        _lib.stream_ptr(out.device),
+        bias.data_ptr() if bias is not None else None, _lib.DTYPE_CODES[bias.dtype] if bias is not None else 0,
+        bias.stride(0) if bias is not None else 0, _lib.stream_ptr(out.device),
     )
     _lib.check(code, "grouped_matmul")
     return (table, block_m)
@@ -210,7 +213,6 @@ def fused_experts_impl(
     quantized where it is produced, so its bf16 form [T*topk, I] is never written to memory.
     """
     assert use_fp8_w8a8 and not use_int8_w8a16, "only the fp8 block-quantized branch is implemented on gfx950"
-    assert w1_bias is None and w2_bias is None, "per-expert bias is not supported by the fp8 block branch"
     fused_act = layout == "blocked" and limit is None and alpha is None   # else: silu_and_mul_fwd + quantizer
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
@@ -252,6 +254,7 @@ def fused_experts_impl(
             pairs, cur, a1_scale, expert_to_token_num, expert_to_tokens, expert_to_weights=expert_to_weights,
             expert_weights=w1, expert_to_weights_scale=w1_scale, topk_num=topk_num, out=c1.view(-1, N),
             mul_routed_weight=False, use_fp8_w8a8=True, alloc_tensor_func=alloc_tensor_func, run_config=run_config,
+            bias=w1_bias,
         )
         if fused_act:
             silu_and_mul_post_quant_fwd(c1.view(-1, N), c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128))
@@ -263,7 +266,93 @@ def fused_experts_impl(
             pairs, c2_q.view(-1, N // 2), c2_s.view(-1, N // 2 // 128), expert_to_token_num, expert_to_tokens,
             expert_to_weights=expert_to_weights, expert_weights=w2, expert_to_weights_scale=w2_scale, topk_num=1,
             out=c3.view(-1, w2.shape[1]), mul_routed_weight=True, use_fp8_w8a8=True,
-            alloc_tensor_func=alloc_tensor_func, reused_mblock_infos=reused, run_config=run_config,
+            alloc_tensor_func=alloc_tensor_func, reused_mblock_infos=reused, run_config=run_config, bias=w2_bias,
         )
         moe_sum_reduce(c3, out_hidden_states[begin:end])
     return out_hidden_states
+
+
+def inplace_fused_experts_impl(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    w1_bias: Optional[torch.Tensor] = None,
+    w2_bias: Optional[torch.Tensor] = None,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    layout: str = "blocked",
+    alpha: Optional[float] = None,
+    limit: Optional[float] = None,
+) -> None:
+    """`fused_experts_impl` writing the result over ``hidden_states`` (reference :1118-1154; there it is also
+    registered as ``torch.ops.lightllm.inplace_fused_experts_impl``, which this package leaves to the host)."""
+    fused_experts_impl(
+        hidden_states, w1, w2, topk_weights, topk_ids, inplace=True, use_fp8_w8a8=use_fp8_w8a8,
+        use_int8_w8a16=use_int8_w8a16, w1_bias=w1_bias, w2_bias=w2_bias, w1_scale=w1_scale, w2_scale=w2_scale,
+        a1_scale=a1_scale, a2_scale=a2_scale, layout=layout, alpha=alpha, limit=limit,
+    )
+
+
+def outplace_fused_experts_impl(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    w1_bias: Optional[torch.Tensor] = None,
+    w2_bias: Optional[torch.Tensor] = None,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    layout: str = "blocked",
+    alpha: Optional[float] = None,
+    limit: Optional[float] = None,
+) -> torch.Tensor:
+    """`fused_experts_impl` into a new tensor (reference :1187-1223)."""
+    return fused_experts_impl(
+        hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, use_fp8_w8a8=use_fp8_w8a8,
+        use_int8_w8a16=use_int8_w8a16, w1_bias=w1_bias, w2_bias=w2_bias, w1_scale=w1_scale, w2_scale=w2_scale,
+        a1_scale=a1_scale, a2_scale=a2_scale, layout=layout, alpha=alpha, limit=limit,
+    )
+
+
+def fused_experts(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    inplace: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    w1_bias: Optional[torch.Tensor] = None,
+    w2_bias: Optional[torch.Tensor] = None,
+    layout: str = "blocked",
+    alpha: Optional[float] = None,
+    limit: Optional[float] = None,
+):
+    """What ``FuseMoeTriton`` calls (reference :1258-1290; note the argument order: the scales come before the
+    biases here and after them in the two functions above).  Returns ``hidden_states`` itself when ``inplace``."""
+    if inplace:
+        inplace_fused_experts_impl(
+            hidden_states, w1, w2, topk_weights, topk_ids, use_fp8_w8a8, use_int8_w8a16, w1_bias, w2_bias, w1_scale,
+            w2_scale, a1_scale, a2_scale, layout=layout, alpha=alpha, limit=limit,
+        )
+        return hidden_states
+    return outplace_fused_experts_impl(
+        hidden_states, w1, w2, topk_weights, topk_ids, use_fp8_w8a8, use_int8_w8a16, w1_bias, w2_bias, w1_scale,
+        w2_scale, a1_scale, a2_scale, layout=layout, alpha=alpha, limit=limit,
+    )

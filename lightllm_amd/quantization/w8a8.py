@@ -45,38 +45,43 @@ class FP8w8a8B128QuantizationMethod(QuantizationMethod):
         out: Optional[torch.Tensor] = None,
         use_custom_tensor_mananger: bool = True,
     ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-        qweight = weight_pack.weight.t()            # [K,N] view, strides (1,K)
-        weight_scale = weight_pack.weight_scale.t()  # [K/128, N/128] view, strides (1,K/128)
-        m, k = input_tensor.shape
-        n = qweight.shape[1]
-        alloc_func = self._alloc_func(use_custom_tensor_mananger)
-        qinput_tensor, input_scale = per_token_group_quant_fp8(
-            input_tensor, self.block_size, dtype=qweight.dtype, alloc_func=alloc_func
-        )
+        """The five GEMM operands in the order of `w8a8_block_fp8_matmul`: quantized activations, the [K, N] view
+        of the weight (strides (1, K)), activation scales, the [K/128, N/128] view of the weight scales, and the
+        output (allocated here unless the caller brings one)."""
+        alloc = self._alloc_func(use_custom_tensor_mananger)
+        w_kn, ws_kn = weight_pack.weight.t(), weight_pack.weight_scale.t()
+        x_q, x_s = per_token_group_quant_fp8(input_tensor, self.block_size, dtype=w_kn.dtype, alloc_func=alloc)
         if out is None:
-            out = alloc_func((m, n), dtype=input_tensor.dtype, device=input_tensor.device)
-        return qinput_tensor, qweight, input_scale, weight_scale, out
+            rows, cols = input_tensor.shape[0], w_kn.shape[1]
+            out = alloc((rows, cols), dtype=input_tensor.dtype, device=input_tensor.device)
+        return x_q, w_kn, x_s, ws_kn, out
 
     def _create_weight(
         self, out_dims: Union[int, List[int]], in_dim: int, dtype: torch.dtype, device_id: int, num_experts: int = 1
     ) -> Tuple[WeightPack, List[WeightPack]]:
-        out_dim = sum(out_dims) if isinstance(out_dims, list) else out_dims
-        expert_prefix = (num_experts,) if num_experts > 1 else ()
+        """One e4m3fn [sum(out_dims), in_dim] weight with its [.. // 128, .. // 128] fp32 scales (a leading expert
+        axis when num_experts > 1), and one view pair per fused sub-weight, cut along the output rows."""
+        b = self.block_size
+        parts = list(out_dims) if isinstance(out_dims, (list, tuple)) else [out_dims]
+        rows = sum(parts)
+        lead = (num_experts,) if num_experts > 1 else ()
         device = torch.device("cuda", device_id)
-        weight = torch.empty(expert_prefix + (out_dim, in_dim), dtype=torch.float8_e4m3fn, device=device)
-        weight_scale = torch.empty(
-            expert_prefix + (out_dim // self.block_size, in_dim // self.block_size), dtype=torch.float32, device=device
+
+        def storage(r: int, c: int, dt: torch.dtype) -> torch.Tensor:
+            return torch.empty(lead + (r, c), dtype=dt, device=device)
+
+        fused = WeightPack(
+            weight=storage(rows, in_dim, torch.float8_e4m3fn),
+            weight_scale=storage(rows // b, in_dim // b, torch.float32),
         )
-        mm_param = WeightPack(weight=weight, weight_scale=weight_scale)
-        dims = out_dims if isinstance(out_dims, list) else [out_dims]
-        mm_param_list = self._split_weight_pack(
-            mm_param,
-            weight_out_dims=dims,
+        views = self._split_weight_pack(
+            fused,
+            weight_out_dims=parts,
             weight_split_dim=-2,
-            weight_scale_out_dims=[d // self.block_size for d in dims],
+            weight_scale_out_dims=[p // b for p in parts],
             weight_scale_split_dim=-2,
         )
-        return mm_param, mm_param_list
+        return fused, views
 
 
 @QUANTMETHODS.register(["fp8w8a8-b128-mi355", "fp8w8a8-b128-triton", "fp8w8a8-b128"], platform="cuda")

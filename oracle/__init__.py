@@ -195,17 +195,21 @@ def moe_align2(num_pairs: int, expert_token_num, block_m: int) -> np.ndarray:
 
 
 def grouped_block_gemm(Xq, Xs, W, Ws, expert_to_token_index, expert_to_weights, expert_token_num,
-                       topk_num: int, mul_routed_weight: bool, bn: int = 128, bk: int = 128, out=None):
-    """-> bf16 bits [num_pairs, N]; rows no pair maps to keep the value they had in ``out`` (zeros if None)."""
+                       topk_num: int, mul_routed_weight: bool, bn: int = 128, bk: int = 128, out=None, bias=None):
+    """-> bf16 bits [num_pairs, N]; rows no pair maps to keep the value they had in ``out`` (zeros if None).
+    ``bias`` fp32 [E, N] is added to the accumulator before the routed weight."""
     Xq, Xs, W, Ws = _c(Xq, np.uint8), _c(Xs, np.float32), _c(W, np.uint8), _c(Ws, np.float32)
     idx, ew, cnt = _c(expert_to_token_index, np.int32), _c(expert_to_weights, np.float32), _c(expert_token_num, np.int32)
     E, N, K = W.shape
     P = idx.shape[1]
     if out is None:
         out = np.zeros((P, N), np.uint16)
+    bias = None if bias is None else _c(bias, np.float32)
+    assert bias is None or bias.shape == (E, N)
     lib().oracle_grouped_block_gemm(
         _p(Xq), _p(Xs), _p(W), _p(Ws), _p(idx), _p(ew), _p(cnt), I64(P), I32(E), I32(topk_num),
-        I64(N), I64(K), I32(bn), I32(bk), I32(1 if mul_routed_weight else 0), _p(out),
+        I64(N), I64(K), I32(bn), I32(bk), I32(1 if mul_routed_weight else 0),
+        _p(bias) if bias is not None else None, _p(out),
     )
     return out
 
@@ -257,7 +261,7 @@ def silu_and_mul_group_quant(x_bf16_bits, group: int = 128):
 
 
 def fused_experts(x_bf16_bits, w1_q, w1_s, w2_q, w2_s, topk_ids, topk_weights, layout="blocked", limit=None,
-                  alpha=None) -> np.ndarray:
+                  alpha=None, w1_bias=None, w2_bias=None) -> np.ndarray:
     """The routed-expert FFN as the reference sequences it (fused_moe/grouped_fused_moe.py:1048-1113):
     routing tables, quantize, gate/up grouped GEMM, silu_and_mul, quantize, down grouped GEMM times the routed
     weight, sum over slots.  x bf16 bits [T,H]; w1 e4m3 bytes [E,2I,H]; w2 [E,H,I] -> bf16 bits [T,H]."""
@@ -267,7 +271,7 @@ def fused_experts(x_bf16_bits, w1_q, w1_s, w2_q, w2_s, topk_ids, topk_weights, l
     E = w1_q.shape[0]
     idx, ew, cnt = moe_align_fused(ids, topk_weights, E)
     xq, xs = group_quant_fp8(x)
-    h1 = grouped_block_gemm(xq, xs, w1_q, w1_s, idx, ew, cnt, topk, False)
+    h1 = grouped_block_gemm(xq, xs, w1_q, w1_s, idx, ew, cnt, topk, False, bias=w1_bias)
     aq, as_ = group_quant_fp8(silu_and_mul_ex(h1, layout, limit, alpha))
-    h3 = grouped_block_gemm(aq, as_, w2_q, w2_s, idx, ew, cnt, 1, True)
+    h3 = grouped_block_gemm(aq, as_, w2_q, w2_s, idx, ew, cnt, 1, True, bias=w2_bias)
     return moe_sum_reduce(h3.reshape(T, topk, -1))

@@ -19,7 +19,8 @@
  *   oracle_block_weight_quant   pinned: torch closed form
  *   oracle_block_gemm*          pinned: unit-scale / one-hot special cases, numpy f64
  *   oracle_moe_align, _align1, _align_fused, _align2   pinned: the reference's own golden vectors
- *   oracle_grouped_block_gemm   pinned: per-expert loop of the dense oracle
+ *   oracle_grouped_block_gemm   pinned: per-expert loop of the dense oracle; the bias term by zero bias (= no bias),
+ *                               zero activations (= bf16(bias * routed weight) exactly) and the torch closed form
  *   oracle_silu_and_mul         pinned: torch closed form (bit-equal but for rare 1-ulp exp differences), special values
  *   oracle_moe_sum_reduce       pinned: exactly summable inputs, torch closed form
  *   oracle_block_weight_dequant pinned: torch closed form, round trip through oracle_block_weight_quant
@@ -368,15 +369,16 @@ void oracle_moe_align2(const int32_t *expert_token_num, int32_t num_experts, int
  * for expert e and slot j < expert_token_num[e]:
  *     idx = expert_to_token_index[e, j]
  *     row = idx / topk_num                      (:587, :619)
- *     out[idx, :] = bf16( blockscaled(Xq[row] . W[e]^T) [* expert_to_weights[e, j]] )   (:709-725)
- * Xq [T,K] bytes, Xs [T,K/bk]; W [E,N,K] bytes, Ws [E, N/bn, K/bk];
+ *     out[idx, :] = bf16( (blockscaled(Xq[row] . W[e]^T) [+ bias[e, :]]) [* expert_to_weights[e, j]] )   (:702-725)
+ * Xq [T,K] bytes, Xs [T,K/bk]; W [E,N,K] bytes, Ws [E, N/bn, K/bk]; bias fp32 [E,N] or NULL (added to the fp32
+ * accumulator before the routed weight, :702-715);
  * out bf16 bits [num_pairs, N].  Rows of `out` that no pair maps to are untouched.
  */
 void oracle_grouped_block_gemm(const uint8_t *Xq, const float *Xs, const uint8_t *W, const float *Ws,
                                const int32_t *expert_to_token_index, const float *expert_to_weights,
                                const int32_t *expert_token_num, int64_t num_pairs, int32_t num_experts,
                                int32_t topk_num, int64_t N, int64_t K, int32_t bn, int32_t bk,
-                               int32_t mul_routed_weight, uint16_t *out) {
+                               int32_t mul_routed_weight, const float *bias, uint16_t *out) {
     init_lut();
     int64_t KB = (K + bk - 1) / bk, NB = (N + bn - 1) / bn;
     for (int32_t e = 0; e < num_experts; ++e) {
@@ -389,6 +391,7 @@ void oracle_grouped_block_gemm(const uint8_t *Xq, const float *Xs, const uint8_t
             for (int64_t n = 0; n < N; ++n) {
                 volatile float v = gemm_element_f32(Xq + row * K, Xs + row * KB, 1, We + n * K,
                                                     Wse + (n / bn) * KB, 1, K, bk);
+                if (bias) v = v + bias[(int64_t)e * N + n];
                 if (mul_routed_weight) v = v * rw;
                 out[(int64_t)idx * N + n] = oracle_f32_to_bf16(v);
             }

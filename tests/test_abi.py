@@ -110,6 +110,20 @@ REFERENCE_SIGNATURES = {
         "(token_num_mul_topk_num, token_inputs, token_input_scale, expert_to_token_num, expert_to_token_index, "
         "expert_to_weights, expert_weights, expert_to_weights_scale, topk_num, out, mul_routed_weight, use_fp8_w8a8, "
         "alloc_tensor_func=torch.empty, reused_mblock_infos=None, run_config=None, bias=None)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "fused_experts_impl"):
+        "(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, use_fp8_w8a8=False, use_int8_w8a16=False, "
+        "w1_bias=None, w2_bias=None, w1_scale=None, w2_scale=None, a1_scale=None, a2_scale=None, "
+        "alloc_tensor_func=torch.empty, run_config=None, layout=blocked, limit=None, alpha=None)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "inplace_fused_experts_impl"):
+        "(hidden_states, w1, w2, topk_weights, topk_ids, use_fp8_w8a8=False, use_int8_w8a16=False, w1_bias=None, "
+        "w2_bias=None, w1_scale=None, w2_scale=None, a1_scale=None, a2_scale=None, layout=blocked, alpha=None, limit=None)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "outplace_fused_experts_impl"):
+        "(hidden_states, w1, w2, topk_weights, topk_ids, use_fp8_w8a8=False, use_int8_w8a16=False, w1_bias=None, "
+        "w2_bias=None, w1_scale=None, w2_scale=None, a1_scale=None, a2_scale=None, layout=blocked, alpha=None, limit=None)",
+    ("lightllm_amd.fused_moe.grouped_fused_moe", "fused_experts"):
+        "(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, use_fp8_w8a8=False, use_int8_w8a16=False, "
+        "w1_scale=None, w2_scale=None, a1_scale=None, a2_scale=None, w1_bias=None, w2_bias=None, layout=blocked, "
+        "alpha=None, limit=None)",
 }
 
 
@@ -178,14 +192,11 @@ def test_operators_refuse_cpu_tensors():
 
 
 def test_shape_table_choices_on_256_compute_units():
-    """The shape -> kernel table for the model linears it was measured on (this container has no GPU: the library
-    plans for 256 compute units).  A change of a rule that moves one of these shapes shows here."""
+    """The shape -> kernel table for the model linears it was measured on, planned for 256 compute units with
+    room for every workspace.  A change of a rule that moves one of these shapes shows here."""
     from lightllm_amd import _lib
 
     lib = _lib.lib()
-    if lib.mi355_device_info(-1, (__import__("ctypes").c_int64 * 8)()) == 0:
-        import pytest
-        pytest.skip("a GPU is visible: the table plans for its own compute-unit count")
     T256, T128, SKINNY, GENERIC, T256x128, STREAMK, XSHARE, ROWS = 1, 2, 3, 4, 5, 8, 9, 10
     expect = {
         (4096, 36864, 7168): T256, (4096, 2112, 7168): T256, (2048, 24576, 1536): T256, (256, 36864, 7168): T256,
@@ -207,5 +218,79 @@ def test_shape_table_choices_on_256_compute_units():
         (512, 1536, 7168): T128, (4096, 7168, 256): T128, (1024, 512, 7168): T128, (256, 4096, 4096): T128,
         (16, 256, 100): GENERIC,
     }
-    got = {shape: lib.mi355_block_fp8_gemm_variant(*shape) for shape in expect}
+    got = {shape: lib.mi355_block_fp8_gemm_plan(*shape, 1 << 32, 256) for shape in expect}
     assert got == expect, {k: (got[k], expect[k]) for k in expect if got[k] != expect[k]}
+
+
+_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS = 1, 2, 3, 4, 5, 8, 9, 10
+
+
+def _sweep_shapes(seed: int, count: int):
+    import random
+
+    rnd = random.Random(seed)
+    model = [(28672, 4096), (4096, 14336), (36864, 7168), (7168, 18432), (2112, 7168), (24576, 1536), (6144, 4096),
+             (5120, 13824), (128256, 4096), (10240, 8192), (7168, 2048), (4096, 7168), (1536, 7168), (512, 7168)]
+    for _ in range(count):
+        if rnd.random() < 0.6:
+            n, k = rnd.choice(model)
+        else:
+            n, k = rnd.randrange(1, 400) * 64, rnd.randrange(1, 150) * 128
+        m = rnd.choice([rnd.randrange(1, 65), rnd.randrange(65, 130), rnd.randrange(129, 385), rnd.randrange(385, 8193)])
+        yield m, n, k
+
+
+def test_auto_never_fails_for_want_of_a_workspace():
+    """Whatever the table picks, an AUTO call without a workspace - or with the fixed scratch of the entry point
+    that allocates nothing - ends in a kernel whose plan needs none (or no more than that): the ROWS128 band
+    129 <= M <= 384 under a long K used to fall through to a stream-K plan that then reported MI355_EWORKSPACE."""
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    scratch = _lib.WS_COUNTER_BYTES + (8 << 20)
+    # the shapes of the report, then a seeded sweep; cus = 0 plans for the current device, whose count
+    # mi355_block_fp8_gemm_workspace_bytes uses as well
+    shapes = [(200, 7168, 18432), (256, 4096, 14336), (300, 4096, 14336), (384, 4096, 14336), (320, 5120, 13824),
+              (128, 7168, 18432), (8, 4096, 14336), (64, 28672, 4096), (512, 7168, 18432)]
+    shapes += list(_sweep_shapes(11, 4000))
+    optional = (_T256, _T128, _T256x128, _XSHARE, _GENERIC)   # run unsplit / one workgroup per tile without one
+    for ws_bytes in (0, scratch):
+        for m, n, k in shapes:
+            v = lib.mi355_block_fp8_gemm_plan(m, n, k, ws_bytes, 0)
+            assert v in (_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS), (m, n, k, v)
+            if v not in optional:
+                need = lib.mi355_block_fp8_gemm_workspace_bytes(m, n, k, v)
+                assert need <= ws_bytes, (m, n, k, v, need, ws_bytes)
+    # with room for everything the plan is the table's own choice
+    for m, n, k in shapes[:200]:
+        assert lib.mi355_block_fp8_gemm_plan(m, n, k, 1 << 34, 0) == lib.mi355_block_fp8_gemm_variant(m, n, k)
+
+
+@pytest.mark.parametrize("cus", [8, 64, 128, 304])
+def test_shape_table_off_256_compute_units(cus):
+    """The table's thresholds are all relative to the compute-unit count but were measured at 256.  On other counts
+    (a partitioned device, another bin) its rules must still hold together: every shape gets a kernel that exists,
+    the weight-streaming kernels keep to their row limits, and a compute-bound shape with whole rounds of
+    256 x 256 tiles gets those tiles."""
+    from lightllm_amd import _lib
+
+    lib = _lib.lib()
+    for m, n, k in _sweep_shapes(cus, 3000):
+        for ws_bytes in (0, 1 << 34):
+            v = lib.mi355_block_fp8_gemm_plan(m, n, k, ws_bytes, cus)
+            assert v in (_T256, _T128, _SKINNY, _T256x128, _STREAMK, _XSHARE, _ROWS), (m, n, k, v)
+            if v in (_SKINNY, _XSHARE):
+                assert m <= 64, (m, n, k, v)
+            if v == _ROWS:
+                assert 16 <= m <= 384, (m, n, k, v)
+            if v in (_T256, _STREAMK, _T256x128):
+                assert m > 64, (m, n, k, v)
+            if m <= 64:
+                assert v in (_SKINNY, _XSHARE, _ROWS, _T128), (m, n, k, v)
+    # whole rounds of 256 x 256 tiles, K long enough to be compute-bound: the ping-pong tiles on every count
+    rounds = 4
+    n = 256 * max(cus // 8, 1)
+    assert lib.mi355_block_fp8_gemm_plan(256 * 8 * rounds, n, 7168, 1 << 34, cus) == _T256
+    # decode rows stream the weights on every count
+    assert lib.mi355_block_fp8_gemm_plan(1, 28672, 4096, 1 << 34, cus) == _SKINNY
+    assert lib.mi355_block_fp8_gemm_plan(8, 4096, 14336, 0, cus) in (_SKINNY, _T128)

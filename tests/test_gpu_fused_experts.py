@@ -40,6 +40,45 @@ def test_fused_experts_vs_oracle(hip, T, E, topk, Hd, I):
     assert (got - want).abs().max() <= 2e-2 * want.abs().max()
 
 
+def test_fused_experts_op_level_callers_and_bias(hip):
+    """fused_experts / inplace_fused_experts_impl / outplace_fused_experts_impl (grouped_fused_moe.py:1118-1290,
+    what FuseMoeTriton calls) give the bits of fused_experts_impl; w1_bias / w2_bias reach both grouped GEMMs
+    (:1082, :1109) and match the oracle's sequence with the same biases."""
+    from lightllm_amd.fused_moe import (fused_experts, fused_experts_impl, inplace_fused_experts_impl,
+                                        outplace_fused_experts_impl)
+
+    print("fused_experts op-level callers, bias", flush=True)
+    T, E, topk, Hd, I = 160, 8, 2, 512, 256
+    x = H.activations(T, Hd, seed=61)
+    w1q, w1s, w2q, w2s = _experts(E, I, Hd, seed=62)
+    ids, tw = H.routing(T, E, topk, seed=63)
+    dev = [t.cuda() for t in (w1q, w2q, tw, ids)]
+    kw = dict(use_fp8_w8a8=True, w1_scale=w1s.cuda(), w2_scale=w2s.cuda())
+    base = fused_experts_impl(x.cuda(), *dev, inplace=False, **kw)
+    out = fused_experts(x.cuda(), *dev, inplace=False, **kw)
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    out = outplace_fused_experts_impl(x.cuda(), *dev, **kw)
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    buf = x.cuda()
+    assert inplace_fused_experts_impl(buf, *dev, **kw) is None
+    assert torch.equal(buf.view(torch.int16), base.view(torch.int16))
+    buf = x.cuda()
+    assert fused_experts(buf, *dev, inplace=True, **kw) is buf
+    assert torch.equal(buf.view(torch.int16), base.view(torch.int16))
+
+    b1 = (torch.randn((E, 2 * I), generator=H.gen(64)) * 0.25).to(torch.bfloat16)
+    b2 = (torch.randn((E, Hd), generator=H.gen(65)) * 0.25).float()
+    out = fused_experts(x.cuda(), *dev, inplace=False, w1_bias=b1.cuda(), w2_bias=b2.cuda(), **kw)
+    torch.cuda.synchronize()
+    want = tr.bf16_from_bits(oracle.fused_experts(tr.bits_of(x), tr.bits_of(w1q), w1s.numpy(), tr.bits_of(w2q),
+                                                  w2s.numpy(), ids.numpy(), tw.numpy(), w1_bias=b1.float().numpy(),
+                                                  w2_bias=b2.numpy())).float()
+    got = out.float().cpu()
+    assert tr.cosine(got, want) >= 0.9999
+    assert (got - want).abs().max() <= 2e-2 * want.abs().max()
+    assert not torch.equal(out.view(torch.int16), base.view(torch.int16))
+
+
 @pytest.mark.parametrize("layout,limit,alpha", [("interleaved", None, None), ("blocked", 7.0, 1.702), ("interleaved", 7.0, 1.702)])
 def test_fused_experts_other_activation_forms(hip, layout, limit, alpha):
     """layout / limit / alpha are forwarded to silu_and_mul_fwd as in the reference (grouped_fused_moe.py:1084-1090);

@@ -57,6 +57,34 @@ def _check_small(xq, xs, wq, ws, C):
     assert err <= 2 ** -7, err
 
 
+def test_cpu_reference_config_on_the_gpu(hip):
+    """The CPU reference configuration (M = 32, N = K = 4096, seed 0: activations ~ N(0,1) quantized per 1x128
+    group, weights ~ N(0, 0.02) block-quantized with the reference's load-time quantizer) through the HIP path
+    with the kernel the shape table picks: the whole matrix against the oracle's fp32 per-block form and the
+    float64 dequant-matmul."""
+    from lightllm_amd.quantization import per_token_group_quant_fp8, w8a8_block_fp8_matmul, weight_quant
+
+    print("gemm cpu-reference config M=32 N=4096 K=4096", flush=True)
+    M, N, K = 32, 4096, 4096
+    x = H.activations(M, K, seed=0)
+    w = H.weights(N, K, seed=0)
+    xq, xs = per_token_group_quant_fp8(x.cuda(), 128)
+    wq, ws = weight_quant(w.cuda(), 128)
+    # the operands themselves are the oracle's, bit for bit
+    q_ref, s_ref = oracle.group_quant_fp8(tr.bits_of(x))
+    wq_ref, ws_ref = oracle.block_weight_quant(w.float().numpy())
+    assert np.array_equal(tr.bits_of(xq), q_ref) and np.array_equal(tr.bits_of(xs), s_ref.view(np.uint32))
+    assert np.array_equal(tr.bits_of(wq), wq_ref) and np.array_equal(ws.cpu().numpy(), ws_ref)
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), C, [128, 128]) is C
+    torch.cuda.synchronize()
+    _check_small(xq, xs, wq, ws, C)
+    # and against the reference's own closed form on the CPU (fp8w8a8_block_gemm_kernel.py:213-217 in fp32)
+    ref = tr.dequant_matmul(xq.cpu(), xs.cpu(), wq.cpu(), ws.cpu(), out_dtype=torch.float32)
+    cos, rel = H.gemm_metrics(C.float().cpu(), ref)
+    assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+
+
 @pytest.mark.parametrize("variant", [None, "tile256", "tile256x128", "tile128", "skinny", "rows128", "generic"])
 @pytest.mark.parametrize("M,N,K", [(32, 512, 1024), (1, 256, 512), (64, 384, 2048), (17, 2112, 256)])
 def test_small_vs_oracle(hip, M, N, K, variant):

@@ -133,6 +133,58 @@ def _grouped_case(T, E, topk, N, K, block_m, mul_w, seed):
     assert (got - ref).abs().max() <= ref.abs().max() * 2 ** -7
 
 
+@pytest.mark.parametrize("bias_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("block_m,T,E,N,K", [(16, 40, 12, 384, 512), (64, 300, 6, 200, 256), (128, 700, 5, 384, 512),
+                                             (256, 900, 5, 640, 1152), (256, 2048, 64, 1160, 1152)])
+def test_grouped_bias_vs_oracle(hip, bias_dtype, block_m, T, E, N, K):
+    """The per-expert bias [E, N] (grouped_fused_moe.py:702-707) in every tile that has an epilogue of its own: the
+    ring tiles, the 256-row ping-pong tile and (last case: more tiles than compute units) the 64x512 streaming
+    tile; with and without the routed weight, an n tail, every bias dtype.  bf16 / fp16 biases are widened
+    exactly, so the oracle gets their fp32 values."""
+    from lightllm_amd.fused_moe import grouped_matmul
+    from lightllm_amd.quantization import per_token_group_quant_fp8
+
+    print(f"grouped bias dtype={bias_dtype} block_m={block_m} T={T} E={E} N={N} K={K}", flush=True)
+    topk = 2
+    ids, tw = H.routing(T, E, topk, seed=T + E)
+    idx, w, cnt = _align(ids, tw, E)
+    x = H.activations(T, K, seed=T).cuda()
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    ws = torch.empty((E, -(-N // 128), K // 128), dtype=torch.float32, device="cuda")
+    for e in range(E):
+        wq[e], ws[e] = H.quantized_weights(N, K, seed=900 + e, device="cuda")
+    bias = (torch.randn((E, N), generator=H.gen(N)) * 0.5).to(bias_dtype)
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    P = T * topk
+    for mul_w in (False, True):
+        out = torch.full((P, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, out, mul_routed_weight=mul_w, use_fp8_w8a8=True,
+                       run_config={"BLOCK_SIZE_M": block_m}, bias=bias.cuda())
+        torch.cuda.synchronize()
+        ref_bits = oracle.grouped_block_gemm(tr.bits_of(xq), xs.cpu().numpy(), tr.bits_of(wq), ws.cpu().numpy(),
+                                             idx.cpu().numpy(), w.cpu().numpy(), cnt.cpu().numpy(), topk, mul_w,
+                                             bias=bias.float().numpy())
+        ref = tr.bf16_from_bits(ref_bits).float()
+        got = out.float().cpu()
+        assert not torch.isnan(got).any(), "a routed row was not written"
+        cos, rel = H.gemm_metrics(got, ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (cos, rel)
+        assert (got - ref).abs().max() <= ref.abs().max() * 2 ** -7
+    # a zero bias gives the bits of the launch without one
+    plain = torch.empty((P, N), dtype=torch.bfloat16, device="cuda")
+    zero = torch.empty((P, N), dtype=torch.bfloat16, device="cuda")
+    grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, plain, mul_routed_weight=True, use_fp8_w8a8=True,
+                   run_config={"BLOCK_SIZE_M": block_m})
+    grouped_matmul(P, x, None, cnt, idx, w, wq, ws, topk, zero, mul_routed_weight=True, use_fp8_w8a8=True,
+                   run_config={"BLOCK_SIZE_M": block_m}, bias=torch.zeros((E, N), dtype=bias_dtype, device="cuda"))
+    torch.cuda.synchronize()
+    routed = idx.cpu()[0, : int(cnt.cpu()[0])].long()
+    if routed.numel():
+        # (-0 + 0 = +0: compare values, then bits wherever the plain result is not a negative zero)
+        a, b = plain.cpu()[routed], zero.cpu()[routed]
+        assert torch.equal(a.float(), b.float())
+
+
 @pytest.mark.parametrize("block_m", [None, 16, 32, 64, 128])
 @pytest.mark.parametrize("mul_w,topk", [(False, 4), (True, 1)])
 def test_grouped_vs_oracle(hip, block_m, mul_w, topk):

@@ -91,6 +91,36 @@ def test_into_caller_buffers(hip):
     _check(x.cpu(), xq, xs)
 
 
+@pytest.mark.parametrize("eps", [1e-4, 3.0, 1e-30])
+def test_other_eps_through_the_caller_buffer_entry(hip, eps):
+    """lightllm_per_token_group_quant_fp8 hands its eps to the kernel (fp8act_quant_kernel.py:63-113).  Any value
+    other than 1e-10 takes the kernel with true divisions: groups whose amax lies below the floor (scale = eps/448,
+    no bf16 value), groups above it, an all-zero group, and both scale layouts."""
+    from lightllm_amd.quantization import lightllm_per_token_group_quant_fp8
+
+    print(f"quant eps={eps}", flush=True)
+    g = H.gen(17)
+    M, K = 96, 1024
+    expo = torch.randint(-40, 4, (M, K // 128, 1), generator=g).float()
+    x = (torch.randn((M, K // 128, 128), generator=g) * torch.exp2(expo)).reshape(M, K)
+    x[3, 128:256] = 0.0
+    x = x.to(torch.bfloat16)
+    q_ref, s_ref = oracle.group_quant_fp8(tr.bits_of(x), 128, eps)
+    below = int((s_ref == np.float32(eps) / np.float32(448.0)).sum())
+    if eps >= 1e-4:
+        assert 0 < below, "the case must hold groups below the floor"
+    if eps == 1e-4:
+        assert below < s_ref.size, "and groups above it"
+    for col_major in (False, True):
+        xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device="cuda")
+        xs = torch.empty((K // 128, M), dtype=torch.float32, device="cuda").t() if col_major else \
+            torch.empty((M, K // 128), dtype=torch.float32, device="cuda")
+        lightllm_per_token_group_quant_fp8(x.cuda(), 128, xq, xs, eps=eps)
+        torch.cuda.synchronize()
+        assert np.array_equal(tr.bits_of(xq), q_ref)
+        assert np.array_equal(tr.bits_of(xs.contiguous()), s_ref.view(np.uint32))
+
+
 def test_full_size_properties(hip):
     """The bandwidth config [16384,7168] with outliers and a zero row: bit-exact on a row sample, and
     size-independent properties on the whole tensor."""

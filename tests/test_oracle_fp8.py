@@ -283,6 +283,38 @@ def test_grouped_gemm_is_a_per_expert_loop_of_the_dense_oracle():
             assert np.array_equal(out[pair], oracle.f32_to_bf16(c32[0]))
 
 
+def test_grouped_gemm_bias_term():
+    """The per-expert bias (grouped_fused_moe.py:702-715: added to the fp32 accumulator, then the routed weight):
+    a zero bias is no bias; with all-zero activations the output is bf16(bias * routed weight) exactly; and in
+    general it equals the unbiased fp32 result plus the bias, in fp32, times the weight."""
+    T, E, topk, N, K = 20, 4, 2, 140, 256
+    ids, tw = H.routing(T, E, topk, seed=52)
+    idx, ew, cnt = oracle.moe_align_fused(ids.numpy(), tw.numpy(), E)
+    xq, xs = oracle.group_quant_fp8(tr.bits_of(H.activations(T, K, seed=53)))
+    Wq = np.empty((E, N, K), np.uint8)
+    Ws = np.empty((E, 2, 2), np.float32)
+    for e in range(E):
+        Wq[e], Ws[e] = oracle.block_weight_quant(H.weights(N, K, seed=70 + e).float().numpy())
+    bias = torch.randn((E, N), generator=H.gen(54)).numpy().astype(np.float32)
+    flat_e, flat_w = ids.numpy().ravel(), tw.numpy().ravel()
+    for mul in (False, True):
+        plain = oracle.grouped_block_gemm(xq, xs, Wq, Ws, idx, ew, cnt, topk, mul)
+        assert np.array_equal(oracle.grouped_block_gemm(xq, xs, Wq, Ws, idx, ew, cnt, topk, mul,
+                                                        bias=np.zeros_like(bias)), plain)
+        zq, zs = oracle.group_quant_fp8(np.zeros((T, K), np.uint16))
+        only = oracle.grouped_block_gemm(zq, zs, Wq, Ws, idx, ew, cnt, topk, mul, bias=bias)
+        want = bias[flat_e] * (flat_w[:, None] if mul else np.float32(1.0))
+        assert np.array_equal(only, oracle.f32_to_bf16(want.astype(np.float32)))
+        got = oracle.grouped_block_gemm(xq, xs, Wq, Ws, idx, ew, cnt, topk, mul, bias=bias)
+        for pair in range(T * topk):
+            e, row = flat_e[pair], pair // topk
+            _, c32 = oracle.block_gemm(xq[row:row + 1], xs[row:row + 1], Wq[e], Ws[e], want_f32=True)
+            c32 = c32[0] + bias[e]
+            if mul:
+                c32 = c32 * flat_w[pair]
+            assert np.array_equal(got[pair], oracle.f32_to_bf16(c32.astype(np.float32)))
+
+
 # ---- the steps between and after the two expert GEMMs --------------------------------------------------------
 def test_silu_and_mul_special_values():
     """silu(0) = 0, silu(g) = g for large g (1 + exp(-g) rounds to 1), silu(g) = -0 for g << 0, silu(1) known."""
