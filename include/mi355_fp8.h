@@ -122,6 +122,10 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
 #define MI355_GEMM_ROWS128 10 /* weight streaming, M <= 384, the activation block of a K step in LDS: 256 weight rows per
                                  workgroup up to 128 rows, 128 beyond; a second launch adds the partial sums when K is shared */
 
+#define MI355_GEMM_SKINNY_CU 11 /* weight streaming, M <= 16: the weight rows cut into one equal share per compute unit,
+                                  one workgroup of 8 waves per share and the whole K (no partial sums between
+                                  workgroups); where N / 16 gives the units 1..8 row blocks each */
+
 #define MI355_WS_COUNTER_BYTES 65536
 
 /* The kernel MI355_GEMM_AUTO picks for a packed, 16-byte aligned problem of this shape on the CURRENT device (one of

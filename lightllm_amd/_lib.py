@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355fp8.so")
 GEMM_AUTO, GEMM_TILE256, GEMM_TILE128, GEMM_SKINNY, GEMM_GENERIC, GEMM_TILE256x128 = 0, 1, 2, 3, 4, 5
 GEMM_TILE256_RING, GEMM_TILE256_ONCE, GEMM_TILE256_STREAMK, GEMM_SKINNY_XSHARE = 6, 7, 8, 9
 GEMM_ROWS128 = 10
+GEMM_SKINNY_CU = 11
 WS_COUNTER_BYTES = 65536
 DTYPE_CODES = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}
 

@@ -4,6 +4,7 @@
 #include "gemm_pp.hpp"
 #include "gemm_small.hpp"
 #include "gemm_stream.hpp"
+#include "gemm_streamcu.hpp"
 #include "gemm_xshare.hpp"
 #include "gemm_rows128.hpp"
 #include "gemm_tile.hpp"
@@ -324,6 +325,62 @@ static int launch_stream_mt(GemmArgs &a, const SkinnyPlan &pl, void *ws, hipStre
     }
 }
 
+// ---- the weight stream cut into one equal share per compute unit (gemm_streamcu.hpp): TNW 16-row blocks per
+// workgroup with TNW = ceil(N / 16 / cus), one workgroup of 8 waves per tile, whole K.  Returns TNW, or 0 where the
+// kernel does not apply: more than 16 rows, more than 5 blocks per unit, tiles that fill under 85 % of the units,
+// fewer than two K steps per wave, offsets past 32 bits or scales that do not fit the LDS.
+static int streamcu_tnw(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t as_m, int cus) {
+    if (M > 16 || cus <= 0) return 0;
+    const int64_t blocks = (N + 15) / 16, KB = K / kBlockK;
+    const int64_t tnw = (blocks + cus - 1) / cus;
+    if (tnw > 5 || KB < 16 || KB > CuStreamCfg<1, 1>::max_steps()) return 0;
+    const int64_t tiles = (blocks + tnw - 1) / tnw;
+    if (tiles * 20 < (int64_t)cus * 17) return 0;
+    if (N * ldw >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32)) return 0;
+    if (8 * ((16 * tnw + 16) * 128) + KB * (17 + 2) * 4 > kMaxLds) return 0;
+    return (int)tnw;
+}
+
+// Where it is ahead of the streaming kernel (M = 1 / 8 / 16, weights rotated past the memory-side cache): wherever
+// that kernel has to share K between workgroups (N = 4096, K = 14336: 12.3 - 13.0 / 12.6 - 13.4 / 13.6 - 14.4 us
+// against 13.4 / 13.7 / 14.9; N = 7168, K = 18432: 23.1 / 23.9 / 25.4 against 26.6 / 28.8 / 30.9), and from three
+// row blocks per unit on, where the 64-row tiles fill their last round badly (N = 14336, K = 4096: 13.4 / 13.5 / 14.0
+// against 14.5 / 15.0 / 16.0; N = 18432, K = 7168: 23.4 / 23.3 / 23.6 against 23.0 / 24.0 / 27.1).  With one or two
+// blocks per unit and K unshared the 16-row tiles of the streaming kernel are ahead (N = 7168, K = 8192: 16.6
+// against 12.9).
+static bool streamcu_pays(int64_t M, int64_t N, int64_t K, int cus) {
+    const int tnw = streamcu_tnw(M, N, K, K, K, K / kBlockK, cus);
+    if (tnw == 0) return false;
+    return skinny_plan(M, N, K, cus).splits > 1 || tnw >= 3;
+}
+
+template <int TNW>
+static int launch_streamcu_as(GemmArgs &a, hipStream_t st) {
+    using Cfg = CuStreamCfg<1, TNW>;
+    constexpr auto kernel_lo = block_fp8_gemm_streamcu_kernel<1, TNW, false>;
+    constexpr auto kernel_hi = block_fp8_gemm_streamcu_kernel<1, TNW, true>;
+    const int lds_bytes = Cfg::lds_bytes(a.K / kBlockK);
+    if (lds_bytes > kMaxLds) return MI355_EUNSUPPORTED;
+    const int tiles = (a.N + Cfg::BN - 1) / Cfg::BN;
+    if (a.M <= 8) {
+        if (!allow_lds<kernel_lo>(kMaxLds)) return MI355_ELAUNCH;
+        return launch(kernel_lo, dim3(tiles), dim3(Cfg::kThreads), lds_bytes, st, a);
+    }
+    if (!allow_lds<kernel_hi>(kMaxLds)) return MI355_ELAUNCH;
+    return launch(kernel_hi, dim3(tiles), dim3(Cfg::kThreads), lds_bytes, st, a);
+}
+
+static int launch_streamcu(GemmArgs &a, int tnw, hipStream_t st) {
+    switch (tnw) {
+        case 1: return launch_streamcu_as<1>(a, st);
+        case 2: return launch_streamcu_as<2>(a, st);
+        case 3: return launch_streamcu_as<3>(a, st);
+        case 4: return launch_streamcu_as<4>(a, st);
+        case 5: return launch_streamcu_as<5>(a, st);
+        default: return MI355_EUNSUPPORTED;
+    }
+}
+
 // ---- the second streaming kernel (activation block shared by the workgroup).  Measured against the first one on
 // the Llama decode shapes it wins only where the first is shortest of registers and N alone fills the device:
 // M = 33..64 with 128-row workgroup tiles (N=28672, K=4096, M=64: 29.7 us against 34.4); with 64-row tiles, few
@@ -637,6 +694,9 @@ static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus);
 //                                                    (M >= 768 and N <= 3072: 256x128 tiles with K shared)
 //   otherwise                                        256x256 ping-pong tiles
 static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_rows128 = true) {
+    // up to 16 rows the per-unit stream also beats the stream with the activation block in LDS where both apply
+    // (N = 18432, K = 7168, M = 16: 23.6 us against 27.5; N = 7168, K = 18432: 25.4 against 27.2)
+    if (streamcu_pays(M, N, K, cus)) return MI355_GEMM_SKINNY_CU;
     if (allow_rows128 && rows128_pays(M, N, K, cus)) return MI355_GEMM_ROWS128;
     if (xshare_pays(M, N, K, cus)) return MI355_GEMM_SKINNY_XSHARE;
     if (M <= 64) return MI355_GEMM_SKINNY;
@@ -758,6 +818,8 @@ static int resolve_auto(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ld
         (N * ldw >= (1ll << 32) || M * lda >= (1ll << 32) || M * as_m >= (1ll << 32) ||
          (N + XshareCfg::BN - 1) / XshareCfg::BN * 4 > MI355_WS_COUNTER_BYTES))
         variant = MI355_GEMM_TILE128;
+    if (variant == MI355_GEMM_SKINNY_CU && streamcu_tnw(M, N, K, lda, ldw, as_m, cus) == 0)
+        variant = MI355_GEMM_SKINNY;
     if (variant == MI355_GEMM_SKINNY &&
         skinny_check(M, N, K, lda, ldw, as_m, cus, ws_usable, ws_bytes) != MI355_OK)
         variant = MI355_GEMM_TILE128;
@@ -945,6 +1007,11 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
                 case 23: return launch_rows128<23>(a, pl, ws, st);
                 default: return launch_rows128<24>(a, pl, ws, st);
             }
+        }
+        case MI355_GEMM_SKINNY_CU: {
+            const int tnw = streamcu_tnw(M, N, K, lda, ldb_n, as_m, cus);
+            if (tnw == 0) return MI355_EUNSUPPORTED;
+            return launch_streamcu(a, tnw, st);
         }
         case MI355_GEMM_SKINNY: {
             const int ok = skinny_check(M, N, K, lda, ldb_n, as_m, cus, ws && ((uintptr_t)ws & 15) == 0, ws_bytes);

@@ -14,7 +14,7 @@ _VARIANTS = {
     None: _lib.GEMM_AUTO, "auto": _lib.GEMM_AUTO, "tile256": _lib.GEMM_TILE256, "tile128": _lib.GEMM_TILE128,
     "skinny": _lib.GEMM_SKINNY, "generic": _lib.GEMM_GENERIC, "tile256x128": _lib.GEMM_TILE256x128,
     "tile256ring": _lib.GEMM_TILE256_RING, "tile256once": _lib.GEMM_TILE256_ONCE,
-    "tile256streamk": _lib.GEMM_TILE256_STREAMK, "xshare": _lib.GEMM_SKINNY_XSHARE, "rows128": _lib.GEMM_ROWS128,
+    "tile256streamk": _lib.GEMM_TILE256_STREAMK, "xshare": _lib.GEMM_SKINNY_XSHARE, "rows128": _lib.GEMM_ROWS128, "streamcu": _lib.GEMM_SKINNY_CU,
 }
 
 

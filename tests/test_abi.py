@@ -65,7 +65,8 @@ def test_pure_host_entry_points():
     assert lib.mi355_grouped_block_m(128 * 16, 128, 3072, 4096) == 16
     assert lib.mi355_grouped_block_m(128 * 32, 128, 3072, 4096) == 256
     assert lib.mi355_block_fp8_gemm_workspace_bytes(4096, 4096, 4096, 0) == 65536  # large M: tile counters only
-    assert lib.mi355_block_fp8_gemm_workspace_bytes(8, 4096, 14336, 0) > 65536
+    assert lib.mi355_block_fp8_gemm_workspace_bytes(32, 4096, 14336, 0) > 65536   # the stream shares K
+    assert lib.mi355_block_fp8_gemm_workspace_bytes(8, 4096, 14336, 0) == 0        # one share per unit, whole K
 
 
 def test_preconditions_are_checked_before_launch():
@@ -197,14 +198,14 @@ def test_shape_table_choices_on_256_compute_units():
     from lightllm_amd import _lib
 
     lib = _lib.lib()
-    T256, T128, SKINNY, GENERIC, T256x128, STREAMK, XSHARE, ROWS = 1, 2, 3, 4, 5, 8, 9, 10
+    T256, T128, SKINNY, GENERIC, T256x128, STREAMK, XSHARE, ROWS, CU = 1, 2, 3, 4, 5, 8, 9, 10, 11
     expect = {
         (4096, 36864, 7168): T256, (4096, 2112, 7168): T256, (2048, 24576, 1536): T256, (256, 36864, 7168): T256,
         (512, 36864, 7168): T256,                       # launched as a full round plus a second launch for the rest
-        (1, 28672, 4096): SKINNY, (8, 4096, 14336): SKINNY, (64, 4096, 14336): SKINNY, (8, 36864, 7168): SKINNY,
+        (1, 28672, 4096): SKINNY, (8, 4096, 14336): CU, (16, 14336, 4096): CU, (1, 7168, 8192): SKINNY, (64, 4096, 14336): SKINNY, (8, 36864, 7168): SKINNY,
         (64, 128256, 4096): XSHARE, (64, 8192, 8192): SKINNY, (64, 16384, 7168): SKINNY,   # 512 / 256 workgroups
         (64, 14336, 4096): ROWS, (48, 10240, 8192): ROWS, (64, 6144, 4096): SKINNY,
-        (16, 7168, 18432): ROWS, (32, 18432, 7168): ROWS, (32, 28672, 4096): SKINNY, (8, 7168, 18432): SKINNY,
+        (16, 7168, 18432): CU, (32, 18432, 7168): ROWS, (32, 28672, 4096): SKINNY, (8, 7168, 18432): CU,
         (16, 36864, 4096): ROWS, (24, 36864, 7168): ROWS, (64, 28672, 4096): ROWS, (100, 7168, 18432): ROWS, (128, 24576, 1536): ROWS,
         (128, 2112, 7168): ROWS, (200, 4096, 14336): ROWS, (384, 4096, 14336): ROWS,
         (192, 36864, 7168): ROWS, (176, 28672, 4096): ROWS, (224, 28672, 4096): T128,   # narrower workgroups up to 208 rows
@@ -222,7 +223,7 @@ def test_shape_table_choices_on_256_compute_units():
     assert got == expect, {k: (got[k], expect[k]) for k in expect if got[k] != expect[k]}
 
 
-_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS = 1, 2, 3, 4, 5, 8, 9, 10
+_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU = 1, 2, 3, 4, 5, 8, 9, 10, 11
 
 
 def _sweep_shapes(seed: int, count: int):
@@ -253,11 +254,11 @@ def test_auto_never_fails_for_want_of_a_workspace():
     shapes = [(200, 7168, 18432), (256, 4096, 14336), (300, 4096, 14336), (384, 4096, 14336), (320, 5120, 13824),
               (128, 7168, 18432), (8, 4096, 14336), (64, 28672, 4096), (512, 7168, 18432)]
     shapes += list(_sweep_shapes(11, 4000))
-    optional = (_T256, _T128, _T256x128, _XSHARE, _GENERIC)   # run unsplit / one workgroup per tile without one
+    optional = (_T256, _T128, _T256x128, _XSHARE, _GENERIC, _CU)   # run unsplit / one workgroup per tile without one
     for ws_bytes in (0, scratch):
         for m, n, k in shapes:
             v = lib.mi355_block_fp8_gemm_plan(m, n, k, ws_bytes, 0)
-            assert v in (_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS), (m, n, k, v)
+            assert v in (_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU), (m, n, k, v)
             if v not in optional:
                 need = lib.mi355_block_fp8_gemm_workspace_bytes(m, n, k, v)
                 assert need <= ws_bytes, (m, n, k, v, need, ws_bytes)
@@ -278,7 +279,9 @@ def test_shape_table_off_256_compute_units(cus):
     for m, n, k in _sweep_shapes(cus, 3000):
         for ws_bytes in (0, 1 << 34):
             v = lib.mi355_block_fp8_gemm_plan(m, n, k, ws_bytes, cus)
-            assert v in (_T256, _T128, _SKINNY, _T256x128, _STREAMK, _XSHARE, _ROWS), (m, n, k, v)
+            assert v in (_T256, _T128, _SKINNY, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU), (m, n, k, v)
+            if v == _CU:
+                assert m <= 16, (m, n, k, v)
             if v in (_SKINNY, _XSHARE):
                 assert m <= 64, (m, n, k, v)
             if v == _ROWS:
@@ -286,11 +289,11 @@ def test_shape_table_off_256_compute_units(cus):
             if v in (_T256, _STREAMK, _T256x128):
                 assert m > 64, (m, n, k, v)
             if m <= 64:
-                assert v in (_SKINNY, _XSHARE, _ROWS, _T128), (m, n, k, v)
+                assert v in (_SKINNY, _XSHARE, _ROWS, _T128, _CU), (m, n, k, v)
     # whole rounds of 256 x 256 tiles, K long enough to be compute-bound: the ping-pong tiles on every count
     rounds = 4
     n = 256 * max(cus // 8, 1)
     assert lib.mi355_block_fp8_gemm_plan(256 * 8 * rounds, n, 7168, 1 << 34, cus) == _T256
     # decode rows stream the weights on every count
     assert lib.mi355_block_fp8_gemm_plan(1, 28672, 4096, 1 << 34, cus) == _SKINNY
-    assert lib.mi355_block_fp8_gemm_plan(8, 4096, 14336, 0, cus) in (_SKINNY, _T128)
+    assert lib.mi355_block_fp8_gemm_plan(8, 4096, 14336, 0, cus) in (_SKINNY, _T128, _CU)

@@ -273,6 +273,60 @@ def test_stream_kernel_random_shapes(hip):
         assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
 
 
+def test_per_unit_stream_kernel(hip):
+    """The weight stream cut into one share per compute unit (M <= 16, one workgroup of 8 waves per tile, whole K):
+    every tile width of 1..5 row blocks - the 48- and 80-row tiles straddle two 128-row scale blocks, whose scales
+    differ -, N tails that cut the last tile, the last block and the vector stores, 16 to 160 K steps, one or two
+    activation loads per step (M <= 8 / M > 8), column-major activation scales, fp16 output; against the torch fp32
+    dequant-matmul, the plain kernel and the float64 oracle, and bit-equal over repeated launches."""
+    from lightllm_amd.quantization import w8a8_block_fp8_matmul
+
+    rng = np.random.default_rng(4242)
+    cus = _lib_cus()
+    cases = []
+    for tnw, frac in [(1, 1.0), (1, 0.88), (2, 1.0), (2, 0.855), (3, 0.9), (4, 1.0), (5, 0.9), (5, 1.0)]:
+        blocks = int(cus * tnw * frac)
+        for tail in (0, -4, -9):
+            cases.append((int(rng.choice([1, 5, 8, 9, 16])), 16 * blocks + tail, int(rng.choice([2048, 4096, 7168, 18432, 20480]))))
+    cases += [(8, 16 * cus, 14336), (16, 16 * cus, 14336), (1, 32 * cus, 2048)]
+    for case, (M, N, K) in enumerate(cases):
+        print(f"gemm per-unit stream case {case}: M={M} N={N} K={K}", flush=True)
+        xq, xs, wq, ws = _prep(M, N, K, seed=6000 + case, device="cuda")
+        c = _run(xq, xs, wq, ws, "streamcu")
+        assert not torch.isnan(c.float()).any()
+        ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+        cos, rel = H.gemm_metrics(c.float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (M, N, K, cos, rel)
+        g = _run(xq, xs, wq, ws, "generic")
+        assert (c.float() - g.float()).abs().max() <= ref.abs().max() * 2 ** -7, (M, N, K)
+        assert torch.equal(c.view(torch.int16), _run(xq, xs, wq, ws, "streamcu").view(torch.int16))
+        rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 4)])
+        cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 60)])
+        ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                              ws.cpu().numpy(), np.arange(len(rows)), cols)
+        got = c[rows][:, cols].float().cpu().double().numpy()
+        assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
+        if case % 5 == 0:
+            assert torch.equal(c, _run(xq, xs.t().contiguous().t(), wq, ws, "streamcu"))
+            h = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), h, [128, 128], run_config={"variant": "streamcu"})
+            torch.cuda.synchronize()
+            assert (h.float() - ref).abs().max() <= ref.abs().max() * 2 ** -9
+    # outside its limits the forced kernel is refused, and the table does not pick it
+    xq, xs, wq, ws = _prep(17, 4096, 4096, seed=1, device="cuda")
+    with pytest.raises(ValueError):
+        _run(xq, xs, wq, ws, "streamcu")
+    xq, xs, wq, ws = _prep(8, 1024, 4096, seed=1, device="cuda")
+    with pytest.raises(ValueError):
+        _run(xq, xs, wq, ws, "streamcu")
+
+
+def _lib_cus():
+    from lightllm_amd import _lib
+
+    return _lib.device_info()["compute_units"]
+
+
 def test_shared_activation_stream_kernel(hip):
     """The streaming kernel whose workgroup shares the activation block (M = 33..64): random shapes with N tails that
     cut a wave's rows, a workgroup's rows and the vector stores, K from one step to 128, against the torch fp32
@@ -363,7 +417,7 @@ def test_rows128_column_major_scales(hip):
                                    (128, 2112, 7168), (200, 7168, 18432), (160, 28672, 4096), (129, 2112, 7168),
                                    (192, 36864, 7168), (208, 24576, 1536),
                                    (200, 6144, 4096), (384, 4096, 14336), (300, 7168, 16384), (48, 24576, 1536),
-                                   (64, 28672, 4096), (24, 36864, 1024), (48, 10240, 8192), (64, 14336, 4096), (16, 7168, 18432), (32, 18432, 7168)])
+                                   (64, 28672, 4096), (24, 36864, 1024), (48, 10240, 8192), (64, 14336, 4096), (24, 7168, 18432), (32, 18432, 7168)])
 def test_rows128_where_the_table_sends_it(hip, M, N, K):
     """Model linears with 33..384 rows that the shape table gives to the weight stream with the activation block in
     LDS."""

@@ -23,7 +23,7 @@ def _replay_matches(fn_eager, make_graph_outputs, replays=4):
         assert torch.equal(again.view(torch.int16), expect.view(torch.int16))
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 12288, 1024), (8, 4096, 14336), (200, 640, 8192), (100, 4096, 14336), (200, 4096, 14336)])
+@pytest.mark.parametrize("M,N,K", [(4096, 12288, 1024), (8, 4096, 14336), (32, 4096, 14336), (200, 640, 8192), (100, 4096, 14336), (200, 4096, 14336)])
 def test_quant_and_gemm_under_graph_capture(hip, M, N, K):
     """Persistent 256x256 launch (768 tiles), split-K stream launch, split-K 128x128 launch, the 256-weight-row
     stream with its second launch that adds the partial sums."""
@@ -111,7 +111,7 @@ def test_graph_survives_workspace_regrowth(hip):
     from lightllm_amd.quantization import per_token_group_quant_fp8, w8a8_block_fp8_matmul
 
     print("graph capture across workspace regrowth", flush=True)
-    M, N, K = 8, 4096, 14336                      # stream kernel, K split over CTAs: uses partials + counters
+    M, N, K = 32, 4096, 14336                     # stream kernel, K split over CTAs: uses partials + counters
     xq, xs = per_token_group_quant_fp8(H.activations(M, K, seed=31).cuda(), 128)
     wq, ws = H.quantized_weights(N, K, seed=32, device="cuda")
     expect = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
@@ -154,7 +154,7 @@ def test_reset_workspace_recovers_dirty_counters(hip):
     from lightllm_amd import _lib
     from lightllm_amd.quantization import per_token_group_quant_fp8, w8a8_block_fp8_matmul
 
-    M, N, K = 8, 4096, 14336
+    M, N, K = 32, 4096, 14336
     xq, xs = per_token_group_quant_fp8(H.activations(M, K, seed=33).cuda(), 128)
     wq, ws = H.quantized_weights(N, K, seed=34, device="cuda")
     expect = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")

@@ -35,7 +35,7 @@ def _call(lib, name, xq, xs, wq, ws, out, variant, workspace=None):
 
 
 # (M, N, K, variant): a K-split stream launch, a smaller one, a split-K 128x128 launch, a persistent 256x256 launch
-CASES = [(16, 4096, 14336, 0), (8, 2048, 7168, 0), (200, 640, 8192, 2), (4096, 8192, 1024, 1)]
+CASES = [(32, 4096, 14336, 0), (24, 2048, 7168, 0), (200, 640, 8192, 2), (4096, 8192, 1024, 1)]
 
 
 def test_noalloc_entry_point_matches_the_workspace_one(hip):
