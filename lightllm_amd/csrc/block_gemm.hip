@@ -48,10 +48,10 @@ static bool chunked_scales_ok(const GemmArgs &a) {
     return a.xs_k == 1 && (a.K / kBlockK) % 8 == 0 && a.xs_m % 4 == 0 && ((uintptr_t)a.Xs & 15) == 0;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8, bool BIAS = false>
 static int launch_tile_as(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
-    constexpr auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE, XS8>;
+    constexpr auto kernel = block_fp8_gemm_tile_kernel<BM, BN, WM, WN, NSTAGE, MODE, XS8, BIAS>;
     const int KB = a.K / kBlockK;
     // chunked scales keep two [BM rows][8 steps] buffers behind the common layout
     const int lds_bytes = XS8 ? ((Cfg::lds_bytes(KB) + 127) & ~127) + 2 * BM * 32 : Cfg::lds_bytes(KB);
@@ -60,17 +60,24 @@ static int launch_tile_as(GemmArgs &a, int grid, hipStream_t st) {
     return launch(kernel, dim3(grid), dim3(Cfg::kThreads), lds_bytes, st, a);
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool BIAS = false>
 static int launch_tile(GemmArgs &a, int grid, hipStream_t st) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
     constexpr bool kFits = ((Cfg::lds_bytes(144) + 127) & ~127) + 2 * BM * 32 <= kMaxLds;  // up to K = 18432
     if constexpr (kFits) {
         if (chunked_scales_ok(a)) {
-            const int r = launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true>(a, grid, st);
+            const int r = launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, true, BIAS>(a, grid, st);
             if (r != MI355_EUNSUPPORTED) return r;
         }
     }
-    return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false>(a, grid, st);
+    return launch_tile_as<BM, BN, WM, WN, NSTAGE, MODE, false, BIAS>(a, grid, st);
+}
+
+// A grouped launch of ring tiles, with or without the per-expert bias.
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+static int launch_grouped_tile(GemmArgs &a, int grid, hipStream_t st) {
+    if (a.bias) return launch_tile<BM, BN, WM, WN, NSTAGE, kGrouped, true>(a, grid, st);
+    return launch_tile<BM, BN, WM, WN, NSTAGE, kGrouped, false>(a, grid, st);
 }
 
 #ifndef MI355_SK_PANEL
@@ -133,9 +140,9 @@ static size_t stream_k_workspace(int groups) {
 // without one every workgroup runs a single tile.  `sk_groups` > 0 asks for the stream-K launch with that many
 // workgroups (dense only; the workspace must hold stream_k_workspace(sk_groups)).  Returns MI355_EUNSUPPORTED
 // when the K range does not fit the kernel's LDS layout.
-template <bool GROUPED, bool SK, bool SC4>
+template <bool GROUPED, bool SK, bool SC4, bool BIAS = false>
 static int launch_pp_as(GemmArgs &a, int grid, int lds_bytes, hipStream_t st) {
-    constexpr auto kernel = block_fp8_gemm_pp_kernel<GROUPED, SK, SC4>;
+    constexpr auto kernel = block_fp8_gemm_pp_kernel<GROUPED, SK, SC4, false, BIAS>;
     if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
     return launch(kernel, dim3(grid), dim3(PPCfg::kThreads), lds_bytes, st, a);
 }
@@ -171,6 +178,11 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, int sk_gro
         a.counters = (uint32_t *)ws;
         per_xcd = cus / 8;
     }
+    if constexpr (GROUPED) {
+        if (a.bias)
+            return sc4 ? launch_pp_as<true, false, true, true>(a, per_xcd * 8, lds_bytes, st)
+                       : launch_pp_as<true, false, false, true>(a, per_xcd * 8, lds_bytes, st);
+    }
     return sc4 ? launch_pp_as<GROUPED, false, true>(a, per_xcd * 8, lds_bytes, st)
                : launch_pp_as<GROUPED, false, false>(a, per_xcd * 8, lds_bytes, st);
 }
@@ -182,6 +194,11 @@ static int launch_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, int sk_gro
 static size_t grouped_workspace(int64_t table_rows) {
     return (size_t)MI355_WS_COUNTER_BYTES + (((size_t)(2 + 2 * table_rows) * 4 + 255) & ~(size_t)255);
 }
+
+template <auto Kernel>
+struct KernelTag {
+    static constexpr auto value = Kernel;
+};
 
 static int launch_grouped_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hipStream_t st) {
     const int KB = a.K / kBlockK;
@@ -197,14 +214,17 @@ static int launch_grouped_pp(GemmArgs &a, void *ws, size_t ws_bytes, int cus, hi
     a.blocks_per_xcd = (a.total_tiles + 7) / 8;
     const int per_xcd = cus / 8;
     a.small_first = per_xcd * 3 / 8;  // measured on the 256-expert routed batch: 8..14 of 32 are within 3 %
-    if (chunked_scales_ok(a)) {
-        constexpr auto kernel = block_fp8_gemm_pp_kernel<true, false, true, true>;
-        if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
+    auto go = [&](auto kernel_tag) {
+        constexpr auto kernel = decltype(kernel_tag)::value;
+        if (!allow_lds<kernel>(kMaxLds)) return (int)MI355_ELAUNCH;
         return launch(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_roles, st, a);
-    }
-    constexpr auto kernel = block_fp8_gemm_pp_kernel<true, false, false, true>;
-    if (!allow_lds<kernel>(kMaxLds)) return MI355_ELAUNCH;
-    return launch(kernel, dim3(per_xcd * 8), dim3(PPCfg::kThreads), lds_roles, st, a);
+    };
+    const bool sc4 = chunked_scales_ok(a);
+    if (a.bias)
+        return sc4 ? go(KernelTag<block_fp8_gemm_pp_kernel<true, false, true, true, true>>{})
+                   : go(KernelTag<block_fp8_gemm_pp_kernel<true, false, false, true, true>>{});
+    return sc4 ? go(KernelTag<block_fp8_gemm_pp_kernel<true, false, true, true>>{})
+               : go(KernelTag<block_fp8_gemm_pp_kernel<true, false, false, true>>{});
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE = kDense>
@@ -1217,10 +1237,10 @@ static int grouped_block_fp8_gemm_impl(const void *Xq, const float *Xs, const vo
     };
     if ((int64_t)table_rows * ((N + 127) / 128) >= (1ll << 31)) return MI355_EUNSUPPORTED;
     switch (block_m) {
-        case 16: return launch_tile<16, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
-        case 32: return launch_tile<32, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
-        case 64: return launch_tile<64, 128, 1, 4, 4, kGrouped>(a, finish(128), st);
-        case 128: return launch_tile<128, 128, 2, 2, 2, kGrouped>(a, finish(128), st);
+        case 16: return launch_grouped_tile<16, 128, 1, 4, 4>(a, finish(128), st);
+        case 32: return launch_grouped_tile<32, 128, 1, 4, 4>(a, finish(128), st);
+        case 64: return launch_grouped_tile<64, 128, 1, 4, 4>(a, finish(128), st);
+        case 128: return launch_grouped_tile<128, 128, 2, 2, 2>(a, finish(128), st);
         case 256:
             finish(256);
             return launch_grouped_pp(a, ws, ws_bytes, device_cus(), st);

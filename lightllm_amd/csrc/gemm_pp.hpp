@@ -81,9 +81,10 @@ struct PPCfg {
     static constexpr int kPartialBytes = BM * BN * 4;  // one fp32 partial tile
 };
 
-template <bool GROUPED, bool SK, bool SC4, bool ROLES = false>
+template <bool GROUPED, bool SK, bool SC4, bool ROLES = false, bool BIAS = false>
 __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p) {
     static_assert(!(GROUPED && SK), "stream-K is a dense launch");
+    static_assert(!BIAS || GROUPED, "the per-expert bias belongs to the grouped launch");
     static_assert(!ROLES || GROUPED, "the small-block tile belongs to the grouped launch");
     using Cfg = PPCfg;
     constexpr int BM = Cfg::BM, TM = Cfg::TM, TN = Cfg::TN, HM = Cfg::HM, WMS = Cfg::WMS, WNS = Cfg::WNS;
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
             if (item >= total_small) break;
             const uint32_t blk = item / pairs_n;
             const v4i row = *(const v4i *)(p.table + (int64_t)small_rows[blk] * 4);
-            grouped_small_tile(p, lds, __builtin_amdgcn_readfirstlane(row[0]), __builtin_amdgcn_readfirstlane(row[1]) * BM,
+            grouped_small_tile<BIAS>(p, lds, __builtin_amdgcn_readfirstlane(row[0]), __builtin_amdgcn_readfirstlane(row[1]) * BM,
                                __builtin_amdgcn_readfirstlane(row[3]), (int)(item - blk * pairs_n) * SmallCfg::BN);
         }
     };
@@ -568,9 +569,8 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
             const int nbase = done.n0 + wave_n * WNS;
             const int32_t *idx_list = GROUPED ? p.e2t_index + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
             const float *w_list = GROUPED ? p.e2t_weight + (int64_t)done.expert * p.num_pairs + done.m0 : nullptr;
-            const bool add_bias = GROUPED && p.bias != nullptr;
-            float bias[4 * TN];
-            if (add_bias) lane_bias<TN>(p, done.expert, nbase, g4, bias);
+            float bias[BIAS ? 4 * TN : 1];
+            if constexpr (BIAS) lane_bias<TN>(p, done.expert, nbase, g4, bias);
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 const int rl = wave_m * WMS + 16 * i + r16;
@@ -588,9 +588,10 @@ __global__ __launch_bounds__(512) void block_fp8_gemm_pp_kernel(const GemmArgs p
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int vv = 0; vv < 4; ++vv)
-                        o[4 * j + vv] =
-                            GROUPED ? (add_bias ? acc[i][j][vv] + bias[4 * j + vv] : acc[i][j][vv]) * rw : acc[i][j][vv];
+                    for (int vv = 0; vv < 4; ++vv) {
+                        if constexpr (BIAS) o[4 * j + vv] = (acc[i][j][vv] + bias[4 * j + vv]) * rw;
+                        else o[4 * j + vv] = GROUPED ? acc[i][j][vv] * rw : acc[i][j][vv];
+                    }
                 if (p.vec_store && nbase + WNS <= p.N) {
 #pragma unroll
                     for (int h = 0; h < TN / 2; ++h)

@@ -39,6 +39,7 @@ struct SmallCfg {
 
 // One tile: expert `expert`, rows [m0, m0 + rows) of its list (rows <= 64), weight rows [n0, n0 + 512).
 // Every wave of the workgroup calls this with the same arguments; on return all LDS reads are complete.
+template <bool BIAS>
 __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *lds, int expert, int m0, int rows, int n0) {
     using Cfg = SmallCfg;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, WNS = Cfg::WNS;
@@ -160,9 +161,8 @@ __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *l
     // n0 + 64*wave + lane_col(g4, 2h) + [0, 8)
     const int nbase = n0 + wave * WNS;
     const float *w_list = p.e2t_weight + (int64_t)expert * p.num_pairs + m0;
-    const bool add_bias = p.bias != nullptr;
-    float bias[4 * TN];
-    if (add_bias) lane_bias<TN>(p, expert, nbase, g4, bias);
+    float bias[BIAS ? 4 * TN : 1];
+    if constexpr (BIAS) lane_bias<TN>(p, expert, nbase, g4, bias);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int rl = 16 * i + r16;
@@ -174,8 +174,10 @@ __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *l
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int vv = 0; vv < 4; ++vv)
-                o[4 * j + vv] = (add_bias ? acc[i][j][vv] + bias[4 * j + vv] : acc[i][j][vv]) * rw;
+            for (int vv = 0; vv < 4; ++vv) {
+                if constexpr (BIAS) o[4 * j + vv] = (acc[i][j][vv] + bias[4 * j + vv]) * rw;
+                else o[4 * j + vv] = acc[i][j][vv] * rw;
+            }
         if (p.vec_store && nbase + WNS <= p.N) {
 #pragma unroll
             for (int h = 0; h < TN / 2; ++h)

@@ -130,7 +130,10 @@ struct TileCfg {
 
 // XS8: the X scales are row-major with 16-byte aligned rows and K/128 % 8 == 0, so they are fetched as
 // [BM rows][8 steps] chunks (one request per 64 half-rows and chunk) instead of one column per step.
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8>
+// BIAS (grouped launches only): p.bias is added to the accumulator before the routed weight.  A template parameter so
+// that the launches without a bias keep their register allocation (sixteen more values live across the epilogue made
+// the 256x256 kernel spill more and run 5 % slower with or without a bias).
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MODE, bool XS8, bool BIAS = false>
 __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const GemmArgs p) {
     using Cfg = TileCfg<BM, BN, WM, WN, NSTAGE>;
     constexpr int kLoads = Cfg::XI + Cfg::WI + (XS8 ? 0 : 1);  // DMA requests per wave and stage
@@ -405,9 +408,8 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
     // ---- epilogue: lane (r16, g4) holds, for each tm, row m = wave_m*WMS + 16*tm + r16 and, for each MFMA block
     // tn, the 4 columns n0 + wave_n*WNS + lane_col(g4, tn) + [0, 4).
     const int nbase = n0 + wave_n * WNS;
-    const bool add_bias = GROUPED && p.bias != nullptr;
-    float bias[4 * TN];
-    if (add_bias) lane_bias<TN>(p, expert, nbase, g4, bias);
+    float bias[BIAS ? 4 * TN : 1];
+    if constexpr (BIAS) lane_bias<TN>(p, expert, nbase, g4, bias);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int rl = wave_m * WMS + 16 * i + r16;
@@ -425,8 +427,10 @@ __global__ __launch_bounds__(WM *WN * 64) void block_fp8_gemm_tile_kernel(const 
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                o[4 * j + v] = GROUPED ? (add_bias ? acc[i][j][v] + bias[4 * j + v] : acc[i][j][v]) * rw : acc[i][j][v];
+            for (int v = 0; v < 4; ++v) {
+                if constexpr (BIAS) o[4 * j + v] = (acc[i][j][v] + bias[4 * j + v]) * rw;
+                else o[4 * j + v] = GROUPED ? acc[i][j][v] * rw : acc[i][j][v];
+            }
         if (p.vec_store && nbase + WNS <= p.N) {
             if constexpr (TN == 1) {
                 *(v2i *)(cp + lane_col<TN>(g4, 0)) = v2i{(int)pack_out2(o[0], o[1], p.out_f16), (int)pack_out2(o[2], o[3], p.out_f16)};
