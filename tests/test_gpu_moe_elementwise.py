@@ -2,9 +2,11 @@
 against the CPU oracle.
 
 Integer/byte bars: moe_sum_reduce and weight_dequant are bit-exact; the fused silu+quant kernel is bit-exact
-against the GPU's own silu_and_mul followed by the oracle quantizer.  silu_and_mul itself goes through exp():
-the kernel and the oracle may differ by an fp32 ulp before the bf16 rounding, so the bar there is "at most one
-bf16 ulp apart, on fewer than 0.1 % of the elements" (tiny magnitudes below 2^-100 are compared by value).
+against the GPU's own silu_and_mul followed by the oracle quantizer.  silu_and_mul itself goes through exp() and a
+division: the kernel and the oracle may differ by an fp32 ulp or two before the first bf16 rounding, so the bar there
+is "fewer than 0.1 % of the elements differ from the oracle, and each of those is what the reference's own sequence
+gives when bf16(silu(gate)) lands on the neighbouring bf16 value" - the product with `up` and its rounding are exact
+in both (tiny magnitudes below 2^-100 are compared by value).
 """
 import numpy as np
 import pytest
@@ -17,13 +19,28 @@ from tests import helpers as H
 pytestmark = pytest.mark.gpu
 
 
-def _silu_close(got_bits: np.ndarray, want_bits: np.ndarray):
+def _silu_close(got_bits: np.ndarray, want_bits: np.ndarray, x: torch.Tensor = None):
+    """`x` (bf16 [M, 2H] = [gate | up], the blocked plain form): elements that differ from the oracle must equal
+    bf16(a' * up) for a' one bf16 step beside the oracle's a = bf16(silu(gate)).  Without `x` (the other forms):
+    at most one bf16 step apart."""
     got, want = got_bits.astype(np.int32), want_bits.astype(np.int32)
     diff = np.abs(got - want)
     tiny = ((got & 0x7FFF) < 0x0D80) & ((want & 0x7FFF) < 0x0D80)   # both |v| < 2^-100
-    assert np.all((diff <= 1) | tiny), f"max bf16 distance {diff[~tiny].max()}"
     frac = float((diff != 0).mean())
     assert frac < 1e-3, f"{frac:.2e} of the elements differ"
+    if x is None:
+        assert np.all((diff <= 1) | tiny), f"max bf16 distance {diff[~tiny].max()}"
+        return
+    Hh = x.shape[1] // 2
+    g, u = x[:, :Hh].double(), x[:, Hh:].float()
+    a = (g / (1.0 + torch.exp(-g))).to(torch.bfloat16)
+    a_bits = a.view(torch.int16).to(torch.int32)
+    ok = torch.from_numpy((diff == 0) | tiny)
+    for step in (-1, 1):
+        beside = (a_bits + step).to(torch.int16).view(torch.bfloat16)
+        cand = (beside.float() * u).to(torch.bfloat16).view(torch.int16).to(torch.int32)
+        ok |= cand == torch.from_numpy(got).to(torch.int32).reshape(cand.shape).to(torch.int16).to(torch.int32)
+    assert bool(ok.all()), f"{int((~ok).sum())} elements are not explained by a neighbouring bf16(silu(gate))"
 
 
 @pytest.mark.parametrize("M,Hh", [(1, 128), (7, 2048), (64, 1024), (300, 1408), (33, 100), (5, 7)])
@@ -35,7 +52,7 @@ def test_silu_and_mul(hip, M, Hh):
     out = torch.empty((M, Hh), dtype=torch.bfloat16, device="cuda")
     silu_and_mul_fwd(x.cuda(), out)
     torch.cuda.synchronize()
-    _silu_close(tr.bits_of(out), oracle.silu_and_mul(tr.bits_of(x)))
+    _silu_close(tr.bits_of(out), oracle.silu_and_mul(tr.bits_of(x)), x)
 
 
 def test_silu_and_mul_extremes_and_strided_input(hip):
@@ -53,7 +70,7 @@ def test_silu_and_mul_extremes_and_strided_input(hip):
     out = torch.empty((M, Hh), dtype=torch.bfloat16, device="cuda")
     silu_and_mul_fwd(xin, out)
     torch.cuda.synchronize()
-    _silu_close(tr.bits_of(out), oracle.silu_and_mul(tr.bits_of(x)))
+    _silu_close(tr.bits_of(out), oracle.silu_and_mul(tr.bits_of(x)), x)
     assert torch.isfinite(out.float()).all()
 
 
