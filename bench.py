@@ -101,6 +101,17 @@ def make_act(M, K, seed, device, outliers=False):
     return x.to(torch.bfloat16)
 
 
+def measured_traffic(key):
+    """Bytes per launch from profiles/traffic.json (written when the rocprofv3 counter passes of a kernel are
+    summarised into profiles/): fetched + written, or None."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            entry = json.load(f)[key]
+        return float(entry["fetch_bytes"]) + float(entry["write_bytes"])
+    except (OSError, KeyError, ValueError, TypeError):
+        return None
+
+
 def cpu_baseline(M_sample, N, K):
     """The reference's torch dequant+matmul form in fp32 plus its CPU quantizer, timed on the host cores
     on a row sample of the headline workload (full N and K, M_sample of the 4096 rows)."""
@@ -144,7 +155,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true")
-    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|prefill|grouped|moe|copy (for profiling)")
+    ap.add_argument("--only", default=None, help="run just one leg: headline|quant|decode|prefill|grouped|moe|ceiling|copy (for profiling)")
+    ap.add_argument("--shape", default=None,
+                    help="with --only decode / prefill: just the weight of that name (decode: gate_up, down, lm_head, "
+                         "deepseek-v3-gate_up; prefill: gate_up, down, q_a+kv_a, q_b), so that a kernel trace of the "
+                         "run averages one shape's launches only")
+    ap.add_argument("--rows", default=None, help="with --shape: comma-separated M values instead of the leg's own list")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path; this build has no multi-GPU leg (--gpus must be 1)",
@@ -166,6 +182,7 @@ def main():
 
     M, N, K = 4096, 36864, 7168
     run_all = args.only is None
+    rows_only = [int(v) for v in args.rows.split(",")] if args.rows else None
     result = {}
     others = []
 
@@ -229,15 +246,15 @@ def main():
             },
             "roofline": {
                 "bound": "mfma",
-                "kernel": "block_fp8_gemm_pp_kernel<false,false,true,false> (dense 256x256 ping-pong tile, persistent)",
+                "kernel": "block_fp8_gemm_pp_kernel<false,false,true,false,false> (dense 256x256 ping-pong tile, persistent)",
                 "achieved": round(achieved, 1),
                 "peak": FP8_MFMA_PEAK_TFLOPS,
                 "unit": "TFLOP/s",
                 "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
-                # HBM bytes per GEMM launch from rocprofv3 --pmc FETCH_SIZE (x2.0) and WRITE_SIZE (x1.0), factors from
-                # a 1 GiB device copy: 1695.0 MB read + 311.4 MB written
-                # (profiles/gemm_pp_deepseek_gate_up_M4096.md)
-                "traffic": 2.0064e9,
+                # bytes per GEMM launch that cross the L2 (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by
+                # what the same counter reads for a 1 GiB device copy), as the last profile of this kernel recorded
+                # them in profiles/traffic.json; null when that file has no entry for the kernel
+                "traffic": measured_traffic("gemm_pp_deepseek_gate_up_M4096"),
                 "algorithmic_bytes_per_launch": gemm_bytes(M, N, K),
                 "launch_us": round(gemm_us, 2),
                 "launch_us_min_max": [round(gemm_all[0], 2), round(gemm_all[-1], 2)],
@@ -294,10 +311,12 @@ def main():
         # copies (> 600 MB) that no launch finds them in the 256 MB memory-side cache
         for (Nd, Kd, name) in [(28672, 4096, "gate_up"), (4096, 14336, "down"), (128256, 4096, "lm_head"),
                                (36864, 7168, "deepseek-v3 gate_up")]:
+            if args.shape and args.shape != name.replace(" ", "-"):
+                continue
             ncopies = -(-640_000_000 // (Nd * Kd))
             copies = [make_weight(Nd, Kd, 10 + c, dev) for c in range(ncopies)]
             views = [(q.t(), s.t()) for q, s in copies]
-            for Md in (1, 8, 32, 64, 128):
+            for Md in rows_only or (1, 8, 32, 64, 128):
                 xq, xs = per_token_group_quant_fp8(make_act(Md, Kd, 20 + Md, dev), 128)
                 out = torch.empty((Md, Nd), dtype=torch.bfloat16, device=dev)
                 nxt = _rotating(views)
@@ -322,22 +341,38 @@ def main():
         # max(bytes / 8 TB/s, flops / 5.03 PFLOP/s)
         shapes = [(36864, 7168, "gate_up"), (7168, 18432, "down"), (2112, 7168, "q_a+kv_a"), (24576, 1536, "q_b")]
         for (Np, Kp, name) in shapes:
-            wq, ws = make_weight(Np, Kp, 30, dev)
-            wq_t, ws_t = wq.t(), ws.t()
-            for Mp in (128, 192, 256, 512, 1024, 2048, 4096):
-                if name == "gate_up" and Mp == 4096:
+            if args.shape and args.shape != name:
+                continue
+            # a row whose roofline is its byte term is a stream over the weight: like the decode leg it rotates
+            # through enough copies (> 640 MB) that no launch finds the weight in the 256 MB memory-side cache;
+            # the compute-bound rows keep one copy
+            ncopies = -(-640_000_000 // (Np * Kp))
+            copies = [make_weight(Np, Kp, 30 + c, dev) for c in range(ncopies)]
+            views = [(q.t(), s.t()) for q, s in copies]
+            for Mp in rows_only or (128, 192, 256, 512, 1024, 2048, 4096):
+                if name == "gate_up" and Mp == 4096 and not args.shape:
                     continue  # the headline
+                flops = 2.0 * Mp * Np * Kp
+                nbytes = gemm_bytes(Mp, Np, Kp)
+                byte_bound = nbytes / HBM_PEAK_GBS / 1e3 > flops / FP8_MFMA_PEAK_TFLOPS / 1e6
                 xq, xs = per_token_group_quant_fp8(make_act(Mp, Kp, 31, dev), 128)
                 out = torch.empty((Mp, Np), dtype=torch.bfloat16, device=dev)
-                us = _time_calls(lambda: w8a8_block_fp8_matmul(xq, wq_t, xs, ws_t, out, [128, 128]), 10, 3, batches=5)
-                flops = 2.0 * Mp * Np * Kp
+                nxt = _rotating(views if byte_bound else views[:1])
+
+                def call():
+                    q_t, s_t = nxt()
+                    w8a8_block_fp8_matmul(xq, q_t, xs, s_t, out, [128, 128])
+
+                us = _time_calls(call, max(10, 2 * ncopies) if byte_bound else 10, 3, batches=5)
                 tf = flops / us / 1e6
-                roof = roofline_us(flops, gemm_bytes(Mp, Np, Kp))
+                roof = roofline_us(flops, nbytes)
                 others.append({"name": f"deepseek-v3 {name} M={Mp} N={Np} K={Kp}", "us": round(us, 2),
                                "TFLOP/s": round(tf, 1), "frac_mfma": round(tf / FP8_MFMA_PEAK_TFLOPS, 4),
-                               "roofline_us": round(roof, 2), "frac_roofline": round(roof / us, 4)})
+                               "roofline_us": round(roof, 2), "frac_roofline": round(roof / us, 4),
+                               "bound": "hbm" if byte_bound else "mfma",
+                               "rotated_MB": round((ncopies if byte_bound else 1) * Np * Kp / 1e6)})
                 del xq, xs, out
-            del wq, ws, wq_t, ws_t
+            del copies, views
             torch.cuda.empty_cache()
 
     if (run_all and not args.no_others) or args.only == "grouped":
@@ -426,6 +461,29 @@ def main():
                        "GB/s": round(byts / us / 1e3, 1), "frac_hbm": round(byts / us / 1e3 / HBM_PEAK_GBS, 4)})
         del h3, red
         torch.cuda.empty_cache()
+
+    if (run_all and not args.no_others) or args.only == "ceiling":
+        # What the matrix cores give the path's inner arithmetic at most: the 32 fp8 products of a K step per wave on
+        # register-resident operands, accumulated in the matrix core or folded with fp32 scales as the kernels must,
+        # on zero and on random e4m3 operands (the part lowers its clock under load, more so on random data).
+        gen = torch.Generator(device=dev).manual_seed(7)
+        rnd = torch.randint(0, 256, (1 << 17,), generator=gen, device=dev, dtype=torch.uint8)
+        rnd = torch.where((rnd & 0x7F) == 0x7F, rnd ^ 1, rnd)   # no NaN codes
+        zero = torch.zeros_like(rnd)
+        sink = torch.empty((info["compute_units"] * 512,), dtype=torch.float32, device=dev)
+        lib = _lib.lib()
+        iters = 2000
+        for data, dname in ((zero, "zero"), (rnd, "random e4m3")):
+            for fold in (0, 1):
+                def call():
+                    _lib.check(lib.mi355_probe_mfma(data.data_ptr(), sink.data_ptr(), fold, 8, iters,
+                                                    _lib.stream_ptr(dev)), "mi355_probe_mfma")
+                us = _time_calls(call, 3, 2, batches=5)
+                tf = info["compute_units"] * 8 * iters * 32 * 65536.0 / us / 1e6
+                others.append({"name": f"ceiling: fp8 MFMA 16x16x128 {'+ fp32 scale fold' if fold else 'accumulating'}, "
+                                       f"registers only, {dname} operands", "us": round(us, 1), "TFLOP/s": round(tf, 1),
+                               "frac_mfma": round(tf / FP8_MFMA_PEAK_TFLOPS, 4)})
+        del rnd, zero, sink
 
     if args.only == "copy":
         # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size

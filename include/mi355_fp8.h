@@ -317,6 +317,17 @@ int mi355_moe_sum_reduce(const void *in, void *out, int64_t T, int32_t topk, int
 int mi355_block_weight_dequant(const void *q, const float *s, void *out, int64_t N, int64_t K, int32_t block,
                                void *stream);
 
+/* ---- measurement aid ------------------------------------------------------------------------------------------
+ * The inner arithmetic of the block-scaled GEMM with everything else taken away: one workgroup of `waves` (4 or 8)
+ * waves per compute unit, each wave running `iters` times the 32 products v_mfma_f32_16x16x128_f8f6f4 of a
+ * 128 x 64 sub-tile and one K step on operand fragments held in registers - accumulating in the matrix core
+ * (fold = 0), or product by product with the fp32 scale fold of the kernels (fold = 1).  No LDS or memory traffic in
+ * the loop.  `operands`: 128 KiB of e4m3 bytes (32-byte aligned; zeros or random bytes - the clock the part holds
+ * depends on them); `sink`: 4 bytes per thread of the launch (compute units x 64 x waves).  Flops of a launch:
+ * compute units x waves x iters x 32 x 65536.  No counterpart in the reference; bench.py --only ceiling times it to
+ * state what the hardware gives this arithmetic at most. */
+int mi355_probe_mfma(const void *operands, void *sink, int32_t fold, int32_t waves, int32_t iters, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -72,6 +72,7 @@ SIGNATURES = {
     ),
     "mi355_moe_sum_reduce": (_c.c_int, [_vp, _vp, _i64, _i32, _i64, _vp]),
     "mi355_block_weight_dequant": (_c.c_int, [_vp, _vp, _vp, _i64, _i64, _i32, _vp]),
+    "mi355_probe_mfma": (_c.c_int, [_vp, _vp, _i32, _i32, _i32, _vp]),
 }
 
 _lib = None

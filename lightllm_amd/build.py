@@ -7,7 +7,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmi355fp8.so")
-SOURCES = ["capi.hip", "group_quant.hip", "weight_quant.hip", "block_gemm.hip", "moe_align.hip", "moe_elementwise.hip"]
+SOURCES = ["capi.hip", "group_quant.hip", "weight_quant.hip", "block_gemm.hip", "moe_align.hip", "moe_elementwise.hip", "probe.hip"]
 # packed-fp32 VALU ops are switched off for every kernel of this library
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
