@@ -35,10 +35,12 @@ def w8a8_block_fp8_matmul(
     """C = (A * Ascale) @ (B * Bscale), written into ``C`` and returned.
 
     A [M,K] e4m3fn contiguous; B [K,N] e4m3fn (LightLLM passes ``weight.t()``: strides (1,K));
-    Ascale [M, K/128] fp32; Bscale [K/128, ceil(N/128)] fp32; C [M,N] bf16 contiguous.
-    ``run_config`` may be ``{"variant": "auto"|"tile256"|"tile256x128"|"tile128"|"skinny"|"generic"}`` (plus the
-    comparison variants "tile256ring", "tile256once" and "tile256streamk"); the
-    reference's tile dictionaries (BLOCK_M, ...) are accepted and ignored: the shape table is built in.
+    Ascale [M, K/128] fp32; Bscale [K/128, ceil(N/128)] fp32; C [M,N] bf16 or fp16 contiguous (the accumulator is
+    cast to the dtype of ``C``).
+    ``run_config`` may force a kernel: ``{"variant": "auto"|"tile256"|"tile256streamk"|"tile256x128"|"tile128"|
+    "rows128"|"xshare"|"skinny"|"streamcu"|"generic"}`` (plus the comparison variants "tile256ring" and
+    "tile256once"); a forced kernel that cannot run the shape raises ``ValueError``.  The reference's tile
+    dictionaries (BLOCK_M, ...) are accepted and ignored: the shape table is built in.
     """
     assert len(block_size) == 2
     block_k, block_n = block_size[0], block_size[1]
