@@ -148,6 +148,43 @@ def test_graph_survives_workspace_regrowth(hip):
     torch.cuda.current_stream().wait_stream(side)
 
 
+def test_capture_after_a_warm_up_on_another_stream_allocates_nothing(hip):
+    """The reference warms a shape up on the current stream and captures on the side stream that ``torch.cuda.graph``
+    opens by itself (lightllm/common/basemodel/cuda_graph.py, _capture_decode).  The captured call must find the
+    device's workspace sized by the warm-up: no buffer appears during the capture, the allocator hands out nothing,
+    and every replay gives the eager result."""
+    from lightllm_amd import _lib
+    from lightllm_amd.quantization import per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    print("graph capture after a warm-up on the current stream", flush=True)
+    M, N, K = 32, 4096, 14336                     # K shared between workgroups: partials + counters in the workspace
+    xq, xs = per_token_group_quant_fp8(H.activations(M, K, seed=41).cuda(), 128)
+    wq, ws = H.quantized_weights(N, K, seed=42, device="cuda")
+    assert _lib.lib().mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_AUTO) > _lib.WS_COUNTER_BYTES
+    expect = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), expect, [128, 128])          # the warm-up, current stream
+    torch.cuda.synchronize()
+    out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    buffers = {k: v.data_ptr() for k, v in _lib._workspaces.items()}
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):                                                  # torch's own capture stream
+        before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), out, [128, 128])
+        after = torch.cuda.memory_stats()["allocation.all.allocated"]
+    assert after == before, "the captured call allocated device memory"
+    assert {k: v.data_ptr() for k, v in _lib._workspaces.items()} == buffers
+    for r in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), expect.view(torch.int16)), f"replay {r}"
+        eager = torch.empty_like(out)
+        w8a8_block_fp8_matmul(xq, wq.t(), xs, ws.t(), eager, [128, 128])
+        torch.cuda.synchronize()
+        assert torch.equal(eager.view(torch.int16), expect.view(torch.int16))
+
+
 def test_reset_workspace_recovers_dirty_counters(hip):
     """Counter words left non-zero (as an aborted launch would) make a split-K launch wrong; the reset entry point
     restores the invariant."""
