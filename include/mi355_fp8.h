@@ -126,6 +126,10 @@ int mi355_block_weight_quant_fp8(const void *w, int32_t w_dtype, void *q, float 
                                   one workgroup of 8 waves per share and the whole K (no partial sums between
                                   workgroups); where N / 16 gives the units 1..8 row blocks each */
 
+#define MI355_GEMM_ROWS_MTILED 12 /* the kernel of MI355_GEMM_ROWS128 tiled over M as well: one round of tiles of
+                                     16..128 rows x 160..256 weight rows, K unshared, no workspace; for more than 384
+                                     rows on a narrow N (at most 5120 weight rows, K <= 7168) */
+
 #define MI355_WS_COUNTER_BYTES 65536
 
 /* The kernel MI355_GEMM_AUTO picks for a packed, 16-byte aligned problem of this shape on the CURRENT device (one of

@@ -12,6 +12,7 @@ GEMM_AUTO, GEMM_TILE256, GEMM_TILE128, GEMM_SKINNY, GEMM_GENERIC, GEMM_TILE256x1
 GEMM_TILE256_RING, GEMM_TILE256_ONCE, GEMM_TILE256_STREAMK, GEMM_SKINNY_XSHARE = 6, 7, 8, 9
 GEMM_ROWS128 = 10
 GEMM_SKINNY_CU = 11
+GEMM_ROWS_MTILED = 12
 WS_COUNTER_BYTES = 65536
 DTYPE_CODES = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}
 

@@ -670,6 +670,111 @@ static int launch_rows128(GemmArgs &a, const Rows128Plan &pl, void *ws, hipStrea
     return launch_rows128_as<MT, 8>(a, pl, ws, st);
 }
 
+// ---- more rows than that on a narrow N: the same kernel tiled over M as well (tiles_m x tiles_n workgroups in one
+// round, K unshared).  Where N gives few 256-wide tiles the 256x256 launch leaves most units idle (N = 2112: 9 tile
+// columns, 144 tiles at M = 4096, 72 at M = 2048) and its lone round is bound by the latency of its K steps; tiles of
+// 16*mt rows x 32*wv weight rows with mt chosen so that tiles_m * tiles_n just fits the units put a workgroup on
+// (nearly) every unit, each with less to load and to multiply per step.
+struct RowsMPlan {
+    int mt, wv, tiles_m, tiles_n;
+};
+
+static RowsMPlan rowsm_plan(int64_t M, int64_t N, int64_t K, int cus) {
+    RowsMPlan best = {0, 0, 0, 0};
+    if (M <= 0 || cus < 8) return best;
+    const int64_t blocks = (M + 15) / 16;
+    int64_t best_bytes = 0;
+    for (int wv = 8; wv >= 5; --wv) {
+        const int64_t tn = (N + 32 * wv - 1) / (32 * wv);
+        if (tn > cus) continue;
+        const int64_t room = cus / tn;                       // m tiles that fit one round
+        const int64_t mt = (blocks + room - 1) / room;       // row blocks per tile
+        if (mt > 13 || (mt <= 8 && wv == 7)) continue;       // kernels built: 5, 6, 8 waves up to 8 blocks; 5..8 up to 13
+        const int64_t tm = (blocks + mt - 1) / mt;
+        if (tm < 2 || tm * tn * 20 < (int64_t)cus * 11) continue;
+        const int64_t bytes = (16 * mt + 32 * wv) * 128;      // what a unit loads per K step
+        if (best.mt == 0 || mt < best.mt || (mt == best.mt && bytes < best_bytes)) {
+            best = {(int)mt, wv, (int)tm, (int)tn};
+            best_bytes = bytes;
+        }
+    }
+    return best;
+}
+
+static bool rowsm_limits_ok(const RowsMPlan &pl, int64_t M, int64_t K, int64_t lda, int64_t as_m, int64_t as_k) {
+    if (pl.mt == 0) return false;
+    if (M * lda >= (1ll << 32) || M * as_m * 4 >= (1ll << 32) || as_k * 32 >= (1ll << 32)) return false;
+    const int64_t steps = K / kBlockK, ns = pl.mt <= 8 ? 3 : 2, bn = 32 * pl.wv, nblk = (bn + 2 * kBlockN - 2) / kBlockN;
+    const int64_t ring = ns * (16 * pl.mt * 128 + bn * 128);
+    return ((ring + nblk * steps * 4 + 127) & ~127ll) + 2 * 16 * pl.mt * 32 <= 160 * 1024;
+}
+
+// Where it pays (forced against the table's previous choice over N = 1024..8192, K = 1536..14336, M = 400..4096,
+// 256 units).  With K <= 5120 and at most 8 row blocks per tile (three ring slots) it is ahead on every N <= 5120:
+// 1.2 to 2.0 times with up to 4 row blocks (N = 4096, K = 4096, M = 512 / 1024 / 2048: 22.4 / 28.8 / 42.0 us against
+// 27.9 / 36.5 / 47.2; N = 2112, K = 2048, M = 1024: 1.95 times), 1.0 to 1.2 with 5..8; from N = 6144 on and with more
+// row blocks (two slots) the square tiles are level or ahead.  With K = 6144 .. 7168 the panel split of the 256x256
+// tiles shares K between idle units and takes most of the gain: 2..6 row blocks on N <= 3072 are still 1.04 to 1.3
+// times ahead (q_a+kv_a, N = 2112, K = 7168, M = 512 / 1024 / 2048: 1.11 / 1.12 / 1.04), a single block or a wider N
+// is behind.  From K = 8192 on the kernels that share K win everywhere.
+static bool rowsm_pays(int64_t M, int64_t N, int64_t K, int cus) {
+    if (M <= 384) return false;
+    const int64_t KB = K / kBlockK;
+    if (KB < 12 || KB > 56) return false;
+    const RowsMPlan pl = rowsm_plan(M, N, K, cus);
+    if (pl.mt == 0 || pl.mt > 8) return false;
+    if (KB <= 40) return N <= 5120;
+    return pl.mt >= 2 && pl.mt <= 6 && N <= 3072;
+}
+
+template <int MT>
+static int launch_rowsm_mt(GemmArgs &a, const Rows128Plan &pl, hipStream_t st) {
+    if constexpr (MT <= 8) {
+        switch (pl.wv) {
+            case 5: return launch_rows128_as<MT, 5>(a, pl, nullptr, st);
+            case 6: return launch_rows128_as<MT, 6>(a, pl, nullptr, st);
+            case 8: return launch_rows128_as<MT, 8>(a, pl, nullptr, st);
+            default: return MI355_EINVAL;
+        }
+    } else {
+        switch (pl.wv) {
+            case 5: return launch_rows128_as<MT, 5, 2>(a, pl, nullptr, st);
+            case 6: return launch_rows128_as<MT, 6, 2>(a, pl, nullptr, st);
+            case 7: return launch_rows128_as<MT, 7, 2>(a, pl, nullptr, st);
+            case 8: return launch_rows128_as<MT, 8, 2>(a, pl, nullptr, st);
+            default: return MI355_EINVAL;
+        }
+    }
+}
+
+static int launch_rowsm(GemmArgs &a, const RowsMPlan &mp, hipStream_t st) {
+    a.tiles_m = mp.tiles_m;
+    a.tiles_n = mp.tiles_n;
+    a.total_tiles = mp.tiles_m * mp.tiles_n;
+    Rows128Plan pl;
+    pl.wv = mp.wv;
+    pl.bn = 32 * mp.wv;
+    pl.splits = 1;
+    pl.tiles = (a.total_tiles + 7) / 8 * 8;  // the kernel numbers its tiles per XCD
+    pl.tn = 2;
+    switch (mp.mt) {
+        case 1: return launch_rowsm_mt<1>(a, pl, st);
+        case 2: return launch_rowsm_mt<2>(a, pl, st);
+        case 3: return launch_rowsm_mt<3>(a, pl, st);
+        case 4: return launch_rowsm_mt<4>(a, pl, st);
+        case 5: return launch_rowsm_mt<5>(a, pl, st);
+        case 6: return launch_rowsm_mt<6>(a, pl, st);
+        case 7: return launch_rowsm_mt<7>(a, pl, st);
+        case 8: return launch_rowsm_mt<8>(a, pl, st);
+        case 9: return launch_rowsm_mt<9>(a, pl, st);
+        case 10: return launch_rowsm_mt<10>(a, pl, st);
+        case 11: return launch_rowsm_mt<11>(a, pl, st);
+        case 12: return launch_rowsm_mt<12>(a, pl, st);
+        case 13: return launch_rowsm_mt<13>(a, pl, st);
+        default: return MI355_EINVAL;
+    }
+}
+
 static bool fast_layout_ok(const void *A, const void *B, int64_t K, int64_t lda, int64_t ldb_k, int64_t ldb_n) {
     return ldb_k == 1 && K % kBlockK == 0 && lda % 16 == 0 && ldb_n % 16 == 0 && ((uintptr_t)A & 15) == 0 &&
            ((uintptr_t)B & 15) == 0;
@@ -706,6 +811,8 @@ static int64_t n_split_rows(int64_t M, int64_t N, int64_t K, int cus);
 //     workgroups neither cus nor 2 cus)              the same, unless the kernel below would run
 //   33 <= M <= 128, 0.55 cus .. cus tiles of 160,
 //     192 or 256 weight rows with K unshared          the same, workgroups of that width
+//   M > 384, N <= 5120 (3072), K <= 5120 (7168), one
+//     round of tiles of at most 128 (96) rows         the same kernel tiled over M, K unshared
 //   M <= 64                                          weight streaming (M > 32 and N/128 about the unit count: the
 //                                                    kernel that shares the activation block in the workgroup)
 //   few 256x256 tiles, long K                        stream-K (the plain loop would leave most units idle)
@@ -718,6 +825,7 @@ static int pick_variant(int64_t M, int64_t N, int64_t K, int cus, bool allow_row
     // (N = 18432, K = 7168, M = 16: 23.6 us against 27.5; N = 7168, K = 18432: 25.4 against 27.2)
     if (streamcu_pays(M, N, K, cus)) return MI355_GEMM_SKINNY_CU;
     if (allow_rows128 && rows128_pays(M, N, K, cus)) return MI355_GEMM_ROWS128;
+    if (allow_rows128 && rowsm_pays(M, N, K, cus)) return MI355_GEMM_ROWS_MTILED;
     if (xshare_pays(M, N, K, cus)) return MI355_GEMM_SKINNY_XSHARE;
     if (M <= 64) return MI355_GEMM_SKINNY;
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
@@ -826,6 +934,8 @@ static size_t workspace_bytes_for(int64_t M, int64_t N, int64_t K, int32_t varia
 static int resolve_auto(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t as_m, int64_t as_k,
                         bool ws_usable, size_t ws_bytes, int cus) {
     int variant = pick_variant(M, N, K, cus);
+    if (variant == MI355_GEMM_ROWS_MTILED && !rowsm_limits_ok(rowsm_plan(M, N, K, cus), M, K, lda, as_m, as_k))
+        variant = pick_variant(M, N, K, cus, false);
     if (variant == MI355_GEMM_ROWS128 &&
         (!rows128_limits_ok(M, N, K, lda, as_m, as_k, cus) ||
          (rows128_splits(M, N, K, cus) > 1 && (!ws_usable || ws_bytes < rows128_workspace(M, N, K, cus)))))
@@ -1027,6 +1137,11 @@ static int block_fp8_gemm_impl(const void *A, const void *B, const float *As, co
                 case 23: return launch_rows128<23>(a, pl, ws, st);
                 default: return launch_rows128<24>(a, pl, ws, st);
             }
+        }
+        case MI355_GEMM_ROWS_MTILED: {
+            const RowsMPlan mp = rowsm_plan(M, N, K, cus);
+            if (!rowsm_limits_ok(mp, M, K, lda, as_m, as_k)) return MI355_EUNSUPPORTED;
+            return launch_rowsm(a, mp, st);
         }
         case MI355_GEMM_SKINNY_CU: {
             const int tnw = streamcu_tnw(M, N, K, lda, ldb_n, as_m, cus);

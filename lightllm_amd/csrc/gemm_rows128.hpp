@@ -86,14 +86,23 @@ __global__ __launch_bounds__(64 * WV) void block_fp8_gemm_rows128_kernel(const G
     const int r16 = lane & 15, g4 = lane >> 4, sub = lane >> 3;
     const uint32_t pch = (uint32_t)(lane & 7);
 
-    uint32_t tile_n, split = 0;
+    uint32_t tile_n, tile_m = 0, split = 0;
     if constexpr (SPLIT) {
         tile_n = blockIdx.x / (uint32_t)p.splits;
         split = blockIdx.x - tile_n * (uint32_t)p.splits;
+    } else if (p.tiles_m > 1) {
+        // more rows than one block holds: tiles_m x tiles_n tiles, n fastest, one contiguous run per XCD (workgroup
+        // ids go round-robin over the 8 XCDs), so the workgroups that share an L2 share their activation rows
+        const uint32_t per_xcd = gridDim.x >> 3;  // the grid is a multiple of 8
+        const uint32_t logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (logical >= (uint32_t)p.total_tiles) return;
+        tile_m = logical / (uint32_t)p.tiles_n;
+        tile_n = logical - tile_m * (uint32_t)p.tiles_n;
     } else {
         tile_n = blockIdx.x;
     }
     const int n0 = (int)tile_n * Cfg::BN;
+    const int m0 = (int)tile_m * (16 * MT);
     const int KB = p.K / kBlockK;
     int kb_begin = 0, kb_end = KB;
     if constexpr (SPLIT) {
@@ -110,7 +119,7 @@ __global__ __launch_bounds__(64 * WV) void block_fp8_gemm_rows128_kernel(const G
     for (int i = 0; i < NXW; ++i) {
         const int g = (wave + Cfg::kWaves * i) % XG;  // waves beyond the block repeat a group (same bytes)
         const int row = 8 * g + sub;
-        const uint32_t src = (uint32_t)min(row, p.M - 1);
+        const uint32_t src = (uint32_t)min(m0 + row, p.M - 1);
         xoff[i] = src * (uint32_t)p.ldx + (pch ^ swz((uint32_t)row)) * 16u;
         xdst[i] = (uint32_t)g * 1024u;
         sc_row[i] = src * (uint32_t)p.xs_m;
@@ -259,7 +268,7 @@ __global__ __launch_bounds__(64 * WV) void block_fp8_gemm_rows128_kernel(const G
     const int nbase = n0 + wave * WNS;
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int rl = 16 * i + r16;
+        const int rl = m0 + 16 * i + r16;
         if (rl >= p.M) continue;
         float o[4 * TN];
 #pragma unroll

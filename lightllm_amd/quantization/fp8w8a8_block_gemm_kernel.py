@@ -14,7 +14,7 @@ _VARIANTS = {
     None: _lib.GEMM_AUTO, "auto": _lib.GEMM_AUTO, "tile256": _lib.GEMM_TILE256, "tile128": _lib.GEMM_TILE128,
     "skinny": _lib.GEMM_SKINNY, "generic": _lib.GEMM_GENERIC, "tile256x128": _lib.GEMM_TILE256x128,
     "tile256ring": _lib.GEMM_TILE256_RING, "tile256once": _lib.GEMM_TILE256_ONCE,
-    "tile256streamk": _lib.GEMM_TILE256_STREAMK, "xshare": _lib.GEMM_SKINNY_XSHARE, "rows128": _lib.GEMM_ROWS128, "streamcu": _lib.GEMM_SKINNY_CU,
+    "tile256streamk": _lib.GEMM_TILE256_STREAMK, "xshare": _lib.GEMM_SKINNY_XSHARE, "rows128": _lib.GEMM_ROWS128, "streamcu": _lib.GEMM_SKINNY_CU, "rowsm": _lib.GEMM_ROWS_MTILED,
 }
 
 
@@ -38,7 +38,7 @@ def w8a8_block_fp8_matmul(
     Ascale [M, K/128] fp32; Bscale [K/128, ceil(N/128)] fp32; C [M,N] bf16 or fp16 contiguous (the accumulator is
     cast to the dtype of ``C``).
     ``run_config`` may force a kernel: ``{"variant": "auto"|"tile256"|"tile256streamk"|"tile256x128"|"tile128"|
-    "rows128"|"xshare"|"skinny"|"streamcu"|"generic"}`` (plus the comparison variants "tile256ring" and
+    "rows128"|"rowsm"|"xshare"|"skinny"|"streamcu"|"generic"}`` (plus the comparison variants "tile256ring" and
     "tile256once"); a forced kernel that cannot run the shape raises ``ValueError``.  The reference's tile
     dictionaries (BLOCK_M, ...) are accepted and ignored: the shape table is built in.
     """

@@ -198,7 +198,7 @@ def test_shape_table_choices_on_256_compute_units():
     from lightllm_amd import _lib
 
     lib = _lib.lib()
-    T256, T128, SKINNY, GENERIC, T256x128, STREAMK, XSHARE, ROWS, CU = 1, 2, 3, 4, 5, 8, 9, 10, 11
+    T256, T128, SKINNY, GENERIC, T256x128, STREAMK, XSHARE, ROWS, CU, ROWSM = 1, 2, 3, 4, 5, 8, 9, 10, 11, 12
     expect = {
         (4096, 36864, 7168): T256, (4096, 2112, 7168): T256, (2048, 24576, 1536): T256, (256, 36864, 7168): T256,
         (512, 36864, 7168): T256,                       # launched as a full round plus a second launch for the rest
@@ -209,12 +209,13 @@ def test_shape_table_choices_on_256_compute_units():
         (16, 36864, 4096): ROWS, (24, 36864, 7168): ROWS, (64, 28672, 4096): ROWS, (100, 7168, 18432): ROWS, (128, 24576, 1536): ROWS,
         (128, 2112, 7168): ROWS, (200, 4096, 14336): ROWS, (384, 4096, 14336): ROWS,
         (192, 36864, 7168): ROWS, (176, 28672, 4096): ROWS, (224, 28672, 4096): T128,   # narrower workgroups up to 208 rows
-        (300, 28672, 4096): T256, (512, 4096, 4096): T128,
+        (300, 28672, 4096): T256, (512, 4096, 4096): ROWSM, (2048, 4096, 4096): ROWSM, (1024, 1024, 4096): ROWSM,
+        (3072, 4096, 4096): T256, (1024, 6144, 4096): T128, (1024, 4096, 8192): STREAMK,   # more than 8 row blocks, a wider N, a longer K
         (300, 36864, 7168): T256,                       # likewise: a full round and the rest
         (512, 7168, 18432): STREAMK, (2048, 4096, 14336): STREAMK, (1024, 7168, 18432): STREAMK,
-        (2048, 2112, 7168): STREAMK, (512, 4096, 14336): STREAMK,     # the panel split
+        (2048, 2112, 7168): ROWSM, (512, 4096, 14336): STREAMK,     # the panel split
         (240, 7168, 18432): STREAMK, (352, 7168, 18432): STREAMK, (300, 7168, 18432): ROWS,
-        (768, 2112, 7168): T256x128, (512, 5120, 5120): T256x128, (1024, 2112, 7168): STREAMK, (512, 4096, 7168): STREAMK,
+        (768, 2112, 7168): ROWSM, (768, 2112, 8192): T256x128, (600, 5120, 6144): T256x128, (512, 5120, 5120): ROWSM, (1024, 2112, 7168): ROWSM, (512, 4096, 7168): STREAMK,
         (384, 16384, 4096): T128, (512, 16384, 7168): STREAMK, (300, 10240, 8192): ROWS, (384, 10240, 4096): T128,
         (512, 1536, 7168): T128, (4096, 7168, 256): T128, (1024, 512, 7168): T128, (256, 4096, 4096): T128,
         (16, 256, 100): GENERIC,
@@ -223,7 +224,7 @@ def test_shape_table_choices_on_256_compute_units():
     assert got == expect, {k: (got[k], expect[k]) for k in expect if got[k] != expect[k]}
 
 
-_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU = 1, 2, 3, 4, 5, 8, 9, 10, 11
+_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU, _ROWSM = 1, 2, 3, 4, 5, 8, 9, 10, 11, 12
 
 
 def _sweep_shapes(seed: int, count: int):
@@ -254,11 +255,11 @@ def test_auto_never_fails_for_want_of_a_workspace():
     shapes = [(200, 7168, 18432), (256, 4096, 14336), (300, 4096, 14336), (384, 4096, 14336), (320, 5120, 13824),
               (128, 7168, 18432), (8, 4096, 14336), (64, 28672, 4096), (512, 7168, 18432)]
     shapes += list(_sweep_shapes(11, 4000))
-    optional = (_T256, _T128, _T256x128, _XSHARE, _GENERIC, _CU)   # run unsplit / one workgroup per tile without one
+    optional = (_T256, _T128, _T256x128, _XSHARE, _GENERIC, _CU, _ROWSM)   # run unsplit / one workgroup per tile without one
     for ws_bytes in (0, scratch):
         for m, n, k in shapes:
             v = lib.mi355_block_fp8_gemm_plan(m, n, k, ws_bytes, 0)
-            assert v in (_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU), (m, n, k, v)
+            assert v in (_T256, _T128, _SKINNY, _GENERIC, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU, _ROWSM), (m, n, k, v)
             if v not in optional:
                 need = lib.mi355_block_fp8_gemm_workspace_bytes(m, n, k, v)
                 assert need <= ws_bytes, (m, n, k, v, need, ws_bytes)
@@ -279,14 +280,16 @@ def test_shape_table_off_256_compute_units(cus):
     for m, n, k in _sweep_shapes(cus, 3000):
         for ws_bytes in (0, 1 << 34):
             v = lib.mi355_block_fp8_gemm_plan(m, n, k, ws_bytes, cus)
-            assert v in (_T256, _T128, _SKINNY, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU), (m, n, k, v)
+            assert v in (_T256, _T128, _SKINNY, _T256x128, _STREAMK, _XSHARE, _ROWS, _CU, _ROWSM), (m, n, k, v)
+            if v == _ROWSM:
+                assert m > 384 and k <= 7168, (m, n, k, v)
             if v == _CU:
                 assert m <= 16, (m, n, k, v)
             if v in (_SKINNY, _XSHARE):
                 assert m <= 64, (m, n, k, v)
             if v == _ROWS:
                 assert 16 <= m <= 384, (m, n, k, v)
-            if v in (_T256, _STREAMK, _T256x128):
+            if v in (_T256, _STREAMK, _T256x128, _ROWSM):
                 assert m > 64, (m, n, k, v)
             if m <= 64:
                 assert v in (_SKINNY, _XSHARE, _ROWS, _T128, _CU), (m, n, k, v)

@@ -427,6 +427,63 @@ def test_rows128_where_the_table_sends_it(hip, M, N, K):
     assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), _run(xq, xs, wq, ws, "rows128").view(torch.int16))
 
 
+def test_rows_tiled_over_m(hip):
+    """The weight stream with the activation block in LDS, tiled over M as well (more than 384 rows on a narrow N, one
+    round of tiles, K unshared): every row-block count 1..8 on three ring slots and 9..13 on two, 5-, 6-, 7- and
+    8-wave workgroups, ragged last row tiles, N tails that cut a workgroup's rows and the vector stores, K from fewer
+    steps than ring slots to 56 - against the torch fp32 dequant-matmul, the float64 oracle on a sample and the
+    128x128 tile (same products in the same order when that does not share K: bit-equal); twice in a row."""
+    from lightllm_amd import _lib
+
+    rng = np.random.default_rng(31415)
+    cases = [(512, 4096, 4096), (1000, 2112, 4096), (4096, 1024, 1536), (700, 3072, 7168), (3001, 576, 2048),
+             (2048, 4096 - 24, 512), (401, 5120, 640), (4096, 2112, 7168), (1500, 1536 + 4, 256), (2500, 1000, 128),
+             (6000, 1024, 384), (8192, 512, 1024), (1024, 2049, 2048), (3333, 3333, 384),
+             # 7 row blocks; 9 on 7 waves; 11 on 6 waves; 13 on 5 waves (a single column of tiles)
+             (3000, 2112, 1024), (5000, 1568, 512), (44000, 190, 256), (52000, 150, 128)]
+    cases += [(int(rng.integers(385, 5000)), int(rng.integers(3, 160)) * int(rng.choice([1, 8, 32])),
+               int(rng.choice([128, 256, 640, 1024, 2048, 4096]))) for _ in range(12)]
+    lib = _lib.lib()
+    seen = set()
+    for case, (M, N, K) in enumerate(cases):
+        print(f"gemm rows tiled over M case {case}: M={M} N={N} K={K}", flush=True)
+        xq, xs, wq, ws = _prep(M, N, K, seed=6400 + case, device="cuda")
+        try:
+            c = _run(xq, xs, wq, ws, "rowsm").clone()
+        except ValueError:
+            continue                          # no one-round plan for this shape: a forced call is refused
+        seen.add(case)
+        assert not torch.isnan(c.float()).any()
+        assert torch.equal(c, _run(xq, xs, wq, ws, "rowsm"))
+        ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
+        cos, rel = H.gemm_metrics(c.float(), ref)
+        assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (M, N, K, cos, rel)
+        t = _run(xq, xs, wq, ws, "tile128")
+        if lib.mi355_block_fp8_gemm_workspace_bytes(M, N, K, _lib.GEMM_TILE128) == 0:
+            assert torch.equal(c.view(torch.int16), t.view(torch.int16)), (M, N, K)
+        else:
+            assert (c.float() - t.float()).abs().max() <= ref.abs().max() * 2 ** -7, (M, N, K)
+        rows = np.unique(np.r_[0, M - 1, rng.integers(0, M, 6)])
+        cols = np.unique(np.r_[0, N - 1, rng.integers(0, N, 30)])
+        ref64 = oracle.dequant_matmul_sampled(tr.bits_of(xq[rows].contiguous()), xs[rows].cpu().numpy(), tr.bits_of(wq),
+                                              ws.cpu().numpy(), np.arange(len(rows)), cols)
+        got = c[rows][:, cols].float().cpu().double().numpy()
+        assert np.abs(got - ref64).max() <= H.GEMM_MAX_REL * max(np.abs(ref64).max(), 1e-6)
+    assert len(seen) >= 20 and set(range(18)) <= seen, sorted(seen)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 4096, 4096), (1024, 2112, 7168), (2048, 4096, 4096), (768, 3584, 3584),
+                                   (1024, 1024, 4096), (600, 5120, 5120)])
+def test_rows_tiled_over_m_where_the_table_sends_it(hip, M, N, K):
+    print(f"gemm rows tiled over M, table shape M={M} N={N} K={K}", flush=True)
+    from lightllm_amd import _lib
+
+    assert _lib.lib().mi355_block_fp8_gemm_variant(M, N, K) == _lib.GEMM_ROWS_MTILED
+    _check_full(M, N, K, None, seed=M + N % 89)
+    xq, xs, wq, ws = _prep(M, N, K, seed=1)
+    assert torch.equal(_run(xq, xs, wq, ws, None).view(torch.int16), _run(xq, xs, wq, ws, "rowsm").view(torch.int16))
+
+
 def test_unit_scales_is_plain_matmul(hip):
     """All scales 1: the result is the plain product of the fp8 values, exact in fp32 for K=128."""
     print("gemm unit scales", flush=True)
@@ -486,7 +543,7 @@ def test_mid_m_split_k_tiles(hip, M, N, K):
     assert np.abs(got - ref64).max() / np.abs(ref64).max() <= H.GEMM_MAX_REL
 
 
-@pytest.mark.parametrize("M,N,K", [(768, 2112, 7168), (1024, 2112, 7168), (300, 520, 4096)])
+@pytest.mark.parametrize("M,N,K", [(768, 2112, 8192), (1024, 2112, 7168), (300, 520, 4096)])
 def test_256x128_tiles_with_shared_k(hip, M, N, K):
     """256x128 tiles whose K range is shared between workgroups (few tiles, long K): against the torch fp32
     dequant-matmul, the float64 oracle on a sample and the 128x128 tiles; repeated calls agree bit for bit.  The
@@ -661,7 +718,7 @@ def test_generic_strides(hip):
 @pytest.mark.parametrize("variant,M,N,K", [("rows128", 100, 1000, 2048), ("rows128", 300, 640, 4096), ("rows128", 64, 160 * 150, 256),
                                            ("tile128", 200, 520, 4096), ("tile256", 300, 520, 1024), ("tile256x128", 768, 520, 4096),
                                            ("skinny", 20, 1000, 4096), ("xshare", 40, 4096, 1024), ("tile256streamk", 600, 1024, 8192),
-                                           (None, 512, 36864, 256)])
+                                           ("rowsm", 700, 1000, 2048), ("rowsm", 3000, 2112, 512), (None, 512, 36864, 256)])
 def test_padded_rows_through_the_c_abi(hip, variant, M, N, K):
     """Operands whose rows are longer than they need be (lda > K, ldb_n > K, ldc > N, padded scale rows), as a
     caller that slices larger buffers passes them: every fast kernel against its own result on packed operands
