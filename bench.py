@@ -483,6 +483,11 @@ def main():
                 others.append({"name": f"ceiling: fp8 MFMA 16x16x128 {'+ fp32 scale fold' if fold else 'accumulating'}, "
                                        f"registers only, {dname} operands", "us": round(us, 1), "TFLOP/s": round(tf, 1),
                                "frac_mfma": round(tf / FP8_MFMA_PEAK_TFLOPS, 4)})
+                if fold and data is rnd and result.get("roofline"):
+                    # the headline kernel against what its own instruction mix sustains on this box in this run
+                    # (the data-sheet fraction moves with the box's clock under load; this ratio does not)
+                    result["roofline"]["register_only_mix_TFLOPs"] = round(tf, 1)
+                    result["roofline"]["frac_of_register_only_mix"] = round(result["roofline"]["achieved"] / tf, 4)
         del rnd, zero, sink
 
     if args.only == "copy":
