@@ -455,6 +455,8 @@ def test_rows_tiled_over_m(hip):
         seen.add(case)
         assert not torch.isnan(c.float()).any()
         assert torch.equal(c, _run(xq, xs, wq, ws, "rowsm"))
+        if case % 4 == 0:
+            assert torch.equal(c, _run(xq, xs.t().contiguous().t(), wq, ws, "rowsm"))    # column-major activation scales
         ref = tr.dequant_matmul(xq, xs, wq, ws, out_dtype=torch.float32)
         cos, rel = H.gemm_metrics(c.float(), ref)
         assert cos >= H.GEMM_MIN_COS and rel <= H.GEMM_MAX_REL, (M, N, K, cos, rel)
@@ -717,7 +719,7 @@ def test_generic_strides(hip):
 
 @pytest.mark.parametrize("variant,M,N,K", [("rows128", 100, 1000, 2048), ("rows128", 300, 640, 4096), ("rows128", 64, 160 * 150, 256),
                                            ("tile128", 200, 520, 4096), ("tile256", 300, 520, 1024), ("tile256x128", 768, 520, 4096),
-                                           ("skinny", 20, 1000, 4096), ("xshare", 40, 4096, 1024), ("tile256streamk", 600, 1024, 8192),
+                                           ("skinny", 20, 1000, 4096), ("streamcu", 12, 4096, 4096), ("xshare", 40, 4096, 1024), ("tile256streamk", 600, 1024, 8192),
                                            ("rowsm", 700, 1000, 2048), ("rowsm", 3000, 2112, 512), (None, 512, 36864, 256)])
 def test_padded_rows_through_the_c_abi(hip, variant, M, N, K):
     """Operands whose rows are longer than they need be (lda > K, ldb_n > K, ldc > N, padded scale rows), as a
@@ -798,6 +800,7 @@ def test_quant_method_apply(hip):
                                            ("tile256x128", 260, 300, 256), ("skinny", 9, 1000, 2048), ("skinny", 40, 4100, 4096),
                                            ("xshare", 50, 4096, 1024), ("tile256streamk", 1000, 2048, 16384),
                                            ("rows128", 100, 1000, 512), ("rows128", 128, 4104, 14336), ("rows128", 250, 1004, 4096),
+                                           ("rowsm", 900, 1004, 1024), ("rowsm", 3000, 2112, 512),
                                            ("generic", 7, 130, 256), (None, 64, 28672, 4096), (None, 1024, 2112, 7168)])
 def test_fp16_output(hip, variant, M, N, K):
     """C in fp16: the fp32 accumulator is cast to the dtype of C (fp8w8a8_block_gemm_kernel.py:78; LightLLM allocates C
