@@ -679,7 +679,7 @@ struct RowsMPlan {
     int mt, wv, tiles_m, tiles_n;
 };
 
-static RowsMPlan rowsm_plan(int64_t M, int64_t N, int64_t K, int cus) {
+static RowsMPlan rowsm_plan(int64_t M, int64_t N, int64_t /*K*/, int cus) {
     RowsMPlan best = {0, 0, 0, 0};
     if (M <= 0 || cus < 8) return best;
     const int64_t blocks = (M + 15) / 16;

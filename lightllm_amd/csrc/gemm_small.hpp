@@ -47,7 +47,7 @@ __device__ __forceinline__ void grouped_small_tile(const GemmArgs &p, uint8_t *l
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, g4 = lane >> 4, sub = lane >> 3;
     const uint32_t pch = (uint32_t)(lane & 7);
-    const int KB = p.K / kBlockK, nchunk = (KB + 7) >> 3;
+    const int KB = p.K / kBlockK;
     const uint32_t lds0 = lds_addr(lds);
 
     const int32_t *idx_list = p.e2t_index + (int64_t)expert * p.num_pairs + m0;
